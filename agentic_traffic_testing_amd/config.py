@@ -444,6 +444,158 @@ HYBRID_PRESETS.update({
 ARCHITECTURES["Soselix"] = SoselixConfig.from_dict
 
 
+# ---------------------------------------------------------------------------------------
+# Semezen: pre-norm decoder on several residual streams (hyper-connections) whose mixers read a
+# token-shifted input; a layer's mixer is sliding-window attention whose values are its keys, or
+# a minGRU recurrence; its feed-forward is a dense GELU layer or a mixture of clamped-GLU experts.
+
+@dataclass(frozen=True)
+class WindowAttentionConfig:
+    """Grouped-query softmax attention with biased q / k projections, values = the projected
+    keys (before rotation and norm), rotate-half positions on the first ``rot_dims`` channels with
+    optional wavelength-dependent frequency scaling ``rot_scaling`` = (factor, low, high,
+    original), weightless per-head RMS norm of q and k after the rotation, a sliding window of
+    ``window`` keys (0: all earlier keys) and an element-wise sigmoid output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: tuple | None = None
+
+
+@dataclass(frozen=True)
+class MinGruConfig:
+    """Element-wise gated recurrence of ``width`` channels whose gates read only the current
+    token."""
+    width: int
+
+
+@dataclass(frozen=True)
+class MoeConfig:
+    """``experts`` clamped-GLU feed-forward layers of width ``ff``; a token runs its ``top`` best
+    by sigmoid router score, the score scaling the expert's input."""
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    act_alpha: float = 1.702
+
+
+@dataclass(frozen=True)
+class SemezenLayerConfig:
+    kind: str                 # "attention" | "mingru"
+    mixer: object = None
+    ff: int = 0               # dense feed-forward width (0: none, or see ``moe``)
+    moe: MoeConfig | None = None
+    ff_act: str = "gelu"      # dense activation: "gelu" (erf) or "gelu_tanh"
+
+
+@dataclass(frozen=True)
+class SemezenConfig:
+    name: str = "semezen"
+    vocab_size: int = 1024
+    hidden_size: int = 256
+    layers: tuple = ()
+    rms_norm_eps: float = 1e-6
+    streams: int = 1
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    max_position_embeddings: int = 1 << 20
+    family: str = "semezen"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @staticmethod
+    def from_dict(c: dict, name: str = "semezen") -> "SemezenConfig":
+        """Parse the checkpoint's config.json (keys: vocab, width, norm.eps, streams,
+        layers[].{type, mixer, mlp}; attention: heads, kv_heads, dim, vdim, scale, mask.size,
+        rot.{dims, base, scaling.{factor, low, high, original}}; mingru: width; mlp: kind dense
+        {ff} or moe {expert.{ff, limit}, router.{experts, top}})."""
+        layers = []
+        for i, L in enumerate(c["layers"]):
+            m, t = L["mixer"], L["type"]
+            if t == "attention":
+                rot = m.get("rot") or {}
+                sc = rot.get("scaling")
+                mc = WindowAttentionConfig(
+                    heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                    window=int((m.get("mask") or {}).get("size") or 0),
+                    rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                    rot_scaling=(float(sc["factor"]), float(sc["low"]), float(sc["high"]),
+                                 float(sc["original"])) if sc else None)
+                if mc.heads % mc.kv_heads:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+                if mc.vdim != mc.dim:
+                    raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
+                if mc.rot_dims % 2 or mc.rot_dims > mc.dim:
+                    raise ValueError(f"layer {i}: rot.dims must be even and <= dim")
+            elif t == "mingru":
+                mc = MinGruConfig(width=int(m["width"]))
+            else:
+                raise ValueError(f"unknown layer type {t!r}")
+            mlp = L.get("mlp")
+            ff, moe, act = 0, None, "gelu"
+            if mlp:
+                kind = str(mlp.get("kind", "dense"))
+                if kind == "dense":
+                    ff, act = int(mlp["ff"]), str(mlp.get("act", "gelu"))
+                    if act not in ("gelu", "gelu_tanh"):
+                        raise ValueError(f"layer {i}: unknown activation {act!r}")
+                elif kind == "moe":
+                    moe = MoeConfig(experts=int(mlp["router"]["experts"]),
+                                    top=int(mlp["router"]["top"]), ff=int(mlp["expert"]["ff"]),
+                                    limit=float(mlp["expert"]["limit"]))
+                    if not 1 <= moe.top <= moe.experts:
+                        raise ValueError(f"layer {i}: router.top must be in [1, experts]")
+                else:
+                    raise ValueError(f"unsupported feed-forward kind {kind!r}")
+            layers.append(SemezenLayerConfig(t, mc, ff, moe, act))
+        return SemezenConfig(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                             layers=tuple(layers), rms_norm_eps=float(c["norm"]["eps"]),
+                             streams=int(c.get("streams", 1)))
+
+
+def semezen_preset(name: str, vocab: int, width: int, ff: int, pattern: str, heads: int,
+                   kv_heads: int, dim: int, window: int, experts: int = 8, top: int = 2,
+                   expert_ff: int = 0, streams: int = 2) -> SemezenConfig:
+    """A Semezen shape for benchmarks and tests: two letters per layer, mixer (``a`` window
+    attention, ``g`` minGRU) then feed-forward (``d`` dense, ``e`` experts, ``-`` none)."""
+    layers = []
+    for j in range(0, len(pattern), 2):
+        mx_, f = pattern[j], pattern[j + 1]
+        mc = (WindowAttentionConfig(heads, kv_heads, dim, dim, dim ** -0.5, window, dim // 2,
+                                    500000.0, (8.0, 1.0, 4.0, 8192.0))
+              if mx_ == "a" else MinGruConfig(heads * dim))
+        layers.append(SemezenLayerConfig(
+            "attention" if mx_ == "a" else "mingru", mc, ff if f == "d" else 0,
+            MoeConfig(experts, top, expert_ff or max(8, ff // max(1, top)), 7.0)
+            if f == "e" else None))
+    return SemezenConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers),
+                         streams=streams)
+
+
+HYBRID_PRESETS.update({
+    "semezen-tiny": semezen_preset("semezen-tiny", 512, 128, 192, "adgeae", 4, 2, 32, 24, 6, 2,
+                                   48, 3),
+    # the "small" Llama preset's geometry (width 1024, 8 q / 2 kv heads of 128, FFN 2816, 4 layers)
+    "semezen-small": semezen_preset("semezen-small", 32768, 1024, 2816, "adgeadge", 8, 2, 128,
+                                    1024, 8, 2, 1408),
+    # Llama-3.2-3B / Llama-3.1-8B layer geometry, one attention + dense and one minGRU + experts
+    "semezen-3b-slice": semezen_preset("semezen-3b-slice", 16384, 3072, 8192, "adge", 24, 8, 128,
+                                       1024, 8, 2, 4096),
+    "semezen-8b-slice": semezen_preset("semezen-8b-slice", 16384, 4096, 14336, "adge", 32, 8, 128,
+                                       1024, 8, 2, 7168),
+})
+ARCHITECTURES["Semezen"] = SemezenConfig.from_dict
+
+
 def resolve_model(model: str) -> tuple[ModelConfig, str | None]:
     """Map a reference-style model id (``meta-llama/Llama-3.1-8B-Instruct``), a preset name
     or a local HF directory (config.json [+ *.safetensors]) to a ModelConfig.

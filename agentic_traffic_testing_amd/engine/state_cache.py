@@ -1,7 +1,8 @@
 """Device side of the hybrid cache: per layer, paged K / V pools for softmax mixers and
 (V pages are stored channel-major, [vdim, block], so the P.V matrix-core operand reads keys
 contiguously) and fixed-size per-sequence state (recurrent matrix state in fp32, convolution tails) for
-recurrent mixers, plus the per-sequence previous token.  The host side - which pages and
+recurrent mixers, the previous token's mixer input of token-shifted layers (fp32), plus the
+per-sequence previous token.  The host side - which pages and
 which state slot a sequence owns - is the native ``BlockManager`` (state slots are handed
 out at admission and returned with the pages).
 
@@ -26,6 +27,7 @@ class LayerCacheSpec:
     conv_channels: int = 0     # > 0: tails [slots, conv_taps - 1, conv_channels]
     conv_taps: int = 0
     kv_from: int = -1          # >= 0: no pages of its own, the layer reads that layer's K / V
+    shift_channels: int = 0    # > 0: fp32 [slots, shift_channels], the previous token's mixer input
 
     def page_bytes(self, block_size: int, itemsize: int) -> int:
         if self.kv_from >= 0:
@@ -34,7 +36,8 @@ class LayerCacheSpec:
 
     def slot_bytes(self, itemsize: int) -> int:
         return (self.state_heads * self.state_dim * self.state_vdim * 4
-                + max(0, self.conv_taps - 1) * self.conv_channels * itemsize)
+                + max(0, self.conv_taps - 1) * self.conv_channels * itemsize
+                + self.shift_channels * 4)
 
 
 @dataclass
@@ -43,6 +46,7 @@ class LayerCache:
     v: torch.Tensor | None = None
     state: torch.Tensor | None = None
     conv: torch.Tensor | None = None
+    shift: torch.Tensor | None = None
 
 
 @dataclass
@@ -73,6 +77,9 @@ class HybridCache:
             if sp.conv_channels and sp.conv_taps > 1:
                 lc.conv = torch.zeros(num_slots, sp.conv_taps - 1, sp.conv_channels, dtype=dtype,
                                       device=device)
+            if sp.shift_channels:
+                lc.shift = torch.zeros(num_slots, sp.shift_channels, dtype=torch.float32,
+                                       device=device)
             layers.append(lc)
         return HybridCache(layers, torch.zeros(max(1, num_slots), dtype=torch.int32,
                                                device=device), num_blocks, num_slots, block_size)
@@ -80,7 +87,7 @@ class HybridCache:
     def nbytes(self) -> int:
         seen = {}
         for lc in self.layers:
-            for t in (lc.k, lc.v, lc.state, lc.conv):
+            for t in (lc.k, lc.v, lc.state, lc.conv, lc.shift):
                 if t is not None:
                     seen[t.data_ptr()] = t.numel() * t.element_size()
         return sum(seen.values())

@@ -15,7 +15,11 @@ def model_class(family: str):
         from .soselix import SoselixModel
 
         return SoselixModel
+    if family == "semezen":
+        from .semezen import SemezenModel
+
+        return SemezenModel
     raise ValueError(f"no model registered for family {family!r}")
 
 
-FAMILIES = ("llama", "ledazen", "soselix")
+FAMILIES = ("llama", "ledazen", "soselix", "semezen")

@@ -3,7 +3,9 @@ an optional sink (score 0 or one learned score per head); latent attention's fro
 (absorbed queries, rotate-half positions, compressed K / V pages) and per-head output gate;
 short causal convolutions with carried tails; the gated delta rule and the gated linear
 recurrence (forget-gate and state-space forms) with per-sequence fp32 state; the fp32-residual
-norms, sums and activations around them.
+norms, sums and activations around them; hyper-connection streams, token shift, the minGRU
+recurrence, element-wise gates, GELU, and routed clamped-GLU experts (grouped matrix products
+over rows sorted by expert).
 
 Same device-strict dispatch as ``ops``: GPU tensors run the HIP kernels of
 ``ops/csrc/mixers`` (library ``_atta_mixers.so``, operators ``torch.ops.atta_mix.*``; built on
@@ -77,6 +79,23 @@ def inv_freq(rot_dims: int, base: float, device) -> torch.Tensor:
         torch.float32).to(device)
 
 
+def scaled_inv_freq(rot_dims: int, base: float, scaling, device) -> torch.Tensor:
+    """``inv_freq`` with wavelength-dependent scaling ``(factor, low, high, original)``: a
+    frequency whose wavelength 2 pi / f is shorter than original / high is kept, longer than
+    original / low is divided by factor, between them blended linearly in original / wavelength.
+    float64, rounded once to fp32."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / rot_dims)
+    if scaling is not None:
+        factor, low, high, original = (float(v) for v in scaling)
+        wave = 2.0 * torch.pi / f
+        smooth = (original / wave - low) / (high - low) if high != low else torch.ones_like(f)
+        mid = (1.0 - smooth) * f / factor + smooth * f
+        f = torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor,
+                                                              mid))
+    return f.to(torch.float32).to(device)
+
+
 def embed_pair(table, pair_table, ids, positions, seq_qstart, seq_slot, prev_token, mul_prev,
                mul_cur, buckets):
     if not table.is_cuda:
@@ -108,15 +127,19 @@ def rotary_table(positions, inv_freq_t):
 
 
 def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
-                       k_cache, v_cache, heads, kv_heads, dim, vdim):
+                       k_cache, v_cache, heads, kv_heads, dim, vdim, rotate_half_pairs=False,
+                       norm_last=False):
     """qx / kx / vx: row-strided [T, heads * dim] / [T, kv_heads * dim] / [T, kv_heads * vdim];
-    cos_sin: ``rotary_table`` of the step's positions."""
+    cos_sin: ``rotary_table`` of the step's positions.  ``q_norm`` / ``k_norm`` None: the norm
+    has no weight; ``rotate_half_pairs``: channel i pairs with i + n_freq instead of
+    (2i, 2i + 1); ``norm_last``: rotate first, then norm."""
     if not qx.is_cuda:
         return mref.qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
-                                       cos_sin, k_cache, v_cache, heads, kv_heads, dim, vdim)
+                                       cos_sin, k_cache, v_cache, heads, kv_heads, dim, vdim,
+                                       rotate_half_pairs, norm_last)
     q = torch.empty(qx.shape[0], heads, dim, dtype=qx.dtype, device=qx.device)
     _native().qk_norm_rope_cache(q, qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
-                                 cos_sin, k_cache, v_cache)
+                                 cos_sin, k_cache, v_cache, rotate_half_pairs, norm_last)
     return q
 
 
@@ -128,27 +151,32 @@ def mfma_attention_ok(q, k_cache, v_cache) -> bool:
 
 
 def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff,
-                   scale, sink=True, num_decode=0, max_decode_kv=0, sink_values=None):
+                   scale, sink=True, num_decode=0, max_decode_kv=0, sink_values=None, window=0):
     """Causal attention of every portion's rows over its sequence's pages
     (k_cache [nb, G, BS, d], v_cache [nb, G, dv, BS]).  Sequences [0, num_decode) have one
     query row each and go through the partitioned decode kernel (``max_decode_kv``: their
     longest context, for the grid); ``tile_seq`` / ``tile_qoff`` hold one entry per
     ATTN_TILE_TOKENS query rows of every other portion (sequence index, row offset in it).
-    ``sink_values``: fp32 [H], the sink's (unscaled) score per query head instead of 0."""
+    ``sink_values``: fp32 [H], the sink's (unscaled) score per query head instead of 0.
+    ``window`` > 0: a row at position i sees keys j with 0 <= i - j < window (decode then runs
+    only the partitions that overlap the window)."""
+    window = int(window)
     if not q.is_cuda:
         return mref.sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
-                                   scale, sink, sink_values)
+                                   scale, sink, sink_values, window)
     out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
     part = None
     if num_decode > 0:
         parts = max(1, -(-int(max_decode_kv) // DECODE_PART_TOKENS))
+        if window > 0:   # the window touches at most this many partitions
+            parts = min(parts, -(-window // DECODE_PART_TOKENS) + 1)
         part = torch.empty(num_decode, q.shape[1], parts, v_cache.shape[2] + 2,
                            dtype=torch.float32, device=q.device)
     if tile_seq.shape[0] > 0 or num_decode > 0:
         _native().sink_attention(out, q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
                                  tile_seq, tile_qoff, scale, sink, num_decode,
                                  max(1, int(max_decode_kv)), part,
-                                 mfma_attention_ok(q, k_cache, v_cache), sink_values)
+                                 mfma_attention_ok(q, k_cache, v_cache), sink_values, window)
     return out
 
 
@@ -210,11 +238,13 @@ def add_norm(x, a, sa, b, sb, c, w, eps, one_plus=True, dtype=torch.bfloat16):
     return h
 
 
-def embed_scale(table, ids, scale):
-    """fp32 rows table[id] * scale."""
+def embed_scale(table, ids, scale, copies=0):
+    """fp32 rows table[id] * scale [T, W]; ``copies`` > 0: [T, copies, W], the row that many
+    times (the streams of a multi-stream residual)."""
     if not table.is_cuda:
-        return mref.embed_scale(table, ids, scale)
-    out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+        return mref.embed_scale(table, ids, scale, copies)
+    shape = (ids.shape[0], copies, table.shape[1]) if copies else (ids.shape[0], table.shape[1])
+    out = torch.empty(shape, dtype=torch.float32, device=table.device)
     _native().embed_scale(out, table, ids, float(scale))
     return out
 
@@ -305,3 +335,168 @@ def state_space_scan(x, B, C, dt, dt_bias, a_log, skip, state, positions, seq_qs
     _native().gated_linear_scan(out, state, C, B, x, dt, dt_bias, a_log, skip, positions,
                                 seq_qstart, seq_slot, heads, groups, n_state, vdim, 1)
     return out
+
+
+
+def hyper_norm(xs, w_in, w, eps, dtype=torch.bfloat16):
+    """xs fp32 [T, s, W] (the residual streams): RMS norm with weight ``w`` of
+    u = sum_s w_in[s] xs[:, s] -> [T, W] of ``dtype``.  w_in fp32 [s]."""
+    if not xs.is_cuda:
+        return mref.hyper_norm(xs, w_in, w, eps, dtype)
+    out = torch.empty(xs.shape[0], xs.shape[2], dtype=dtype, device=xs.device)
+    _native().hyper_update_norm(out, xs, None, None, None, w_in, w, eps)
+    return out
+
+
+def hyper_update_norm(xs, y, mix, w_out, w_in_next, w_next, eps, dtype=torch.bfloat16):
+    """Layer boundary of a multi-stream residual in one pass: every stream at once from the old
+    ones, xs[:, t] = sum_s mix[s, t] xs[:, s] + w_out[t] y (fp32, in place), then (unless
+    ``w_next`` is None) the next sub-layer's ``hyper_norm`` of the new streams."""
+    if not xs.is_cuda:
+        mref.hyper_update(xs, y, mix, w_out)
+        return mref.hyper_norm(xs, w_in_next, w_next, eps, dtype) if w_next is not None else None
+    out = (torch.empty(xs.shape[0], xs.shape[2], dtype=dtype, device=xs.device)
+           if w_next is not None else None)
+    _native().hyper_update_norm(out, xs, y, mix, w_out, w_in_next, w_next, eps)
+    return out
+
+
+def token_shift(n, mu, shift_state, positions, seq_qstart, seq_slot, dtype=torch.bfloat16):
+    """h = n + (n_prev - n) * mu with n_prev the previous token's row of n (fp32 [T, W]); the
+    row before a portion is ``shift_state[slot]`` (zeros before position 0), which then takes the
+    portion's last row."""
+    if not n.is_cuda:
+        return mref.token_shift(n, mu, shift_state, positions, seq_qstart, seq_slot, dtype)
+    out = torch.empty(n.shape, dtype=dtype, device=n.device)
+    _native().token_shift(out, n, mu, shift_state, positions, seq_qstart, seq_slot)
+    return out
+
+
+def gate_mul(a, gate, act="sigmoid"):
+    """a [T, N] times sigmoid / SiLU of the row-strided gate [T, N]."""
+    code = ACT_SIGMOID if act == "sigmoid" else ACT_SILU
+    if not a.is_cuda:
+        return mref.gate_mul(a, gate, code)
+    out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+    _native().gate_mul(out, a, gate, code)
+    return out
+
+
+def mingru_scan(z, x, g, state, positions, seq_qstart, seq_slot, dtype=torch.bfloat16):
+    """minGRU over every portion: S = S + sigmoid(z) (c - S), c = x + 1/2 (x >= 0) or sigmoid(x),
+    output S * silu(g) in ``dtype``.  z, x, g row-strided [T, C]; state fp32 [slots, ..., C]
+    advanced in place (zero before position 0)."""
+    if not z.is_cuda:
+        return mref.mingru_scan(z, x, g, state, positions, seq_qstart, seq_slot, dtype)
+    out = torch.empty(z.shape, dtype=dtype, device=z.device)
+    _native().mingru_scan(out, state, z, x, g, positions, seq_qstart, seq_slot)
+    return out
+
+
+def gelu(x, tanh_form=False):
+    if not x.is_cuda:
+        return mref.gelu(x, tanh_form)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _native().gelu(out, x, bool(tanh_form))
+    return out
+
+
+MOE_TILE_ROWS = 64         # rows of one expert per grouped-product tile ...
+MOE_BIG_TILE_ROWS = 128    # ... and for prefill-sized steps on the matrix-core kernel
+MOE_BIG_TILE_PAIRS = 1024  # (row, choice) pairs from which the large tiles are used
+# floating-point operations of a step's expert products (6 pairs ff W) from which the library
+# path runs them (0: never): below it the grouped kernels finish before a host round trip and
+# three launches per expert would
+MOE_LIBRARY_FLOPS = float(os.environ.get("ATTA_MIX_MOE_LIBRARY_FLOPS", "8e11"))
+
+
+def _pair_sum(y, T, k, dtype=None):
+    """y [T * k, W] (a row's k summands adjacent; ``dtype`` or fp32) -> their fp32 sum per row in
+    ``dtype`` (y's own by default)."""
+    dtype = dtype or y.dtype
+    if k == 1 and y.dtype == dtype:
+        return y
+    out = torch.empty(T, y.shape[1], dtype=dtype, device=y.device)
+    _native().pair_sum(out, y.view(T, k, y.shape[1]))
+    return out
+
+
+def clamped_glu(gu, wts, limit, alpha=1.702):
+    """[gate | up] products [R, 2 ff] with the rows' router weights [R] -> activation [R, ff]."""
+    if not gu.is_cuda:
+        return mref.clamped_glu(gu, wts, limit, alpha)
+    out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+    _native().clamped_glu(out, gu, wts, float(limit), float(alpha))
+    return out
+
+
+def _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha):
+    """Prefill-sized steps: rows sorted by expert, then per expert one library product with the
+    stacked [gate; up] matrix, the activation kernel and one library product with the down
+    matrix.  The per-expert row counts come to the host (one synchronisation per call), so this
+    path is not taken while a graph is being recorded."""
+    T, W = h.shape
+    k = idx.shape[1]
+    flat = idx.flatten().long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=w_gu.shape[0]).tolist()
+    xs = h.index_select(0, torch.div(order, k, rounding_mode="floor"))
+    ws = wts.flatten().index_select(0, order)
+    ys = torch.empty(T * k, W, dtype=h.dtype, device=h.device)
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            gu = torch.nn.functional.linear(xs[off:off + c], w_gu[e])
+            torch.mm(clamped_glu(gu, ws[off:off + c], limit, alpha), w_down[e].t(),
+                     out=ys[off:off + c])
+            off += c
+    y = torch.empty_like(ys)
+    y.index_copy_(0, order, ys)
+    return _pair_sum(y, T, k)
+
+
+def moe_route(logits, top):
+    """fp32 router logits [T, E] -> (expert index int32 [T, top], sigmoid score fp32 [T, top]) of
+    every row's ``top`` largest scores (ties: lowest index)."""
+    if not logits.is_cuda:
+        return mref.moe_route(logits, top)
+    T = logits.shape[0]
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    _native().moe_route(idx, wts, logits)
+    return idx, wts
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702):
+    """Routed clamped-GLU experts: out[t] = sum_j W_down[e] act(W_gate[e] (w h_t), W_up[e] (w h_t))
+    over the row's chosen (e, w) = (idx[t, j], wts[t, j]); act(g, u) = g' sigmoid(alpha g')
+    (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit).  w_gu [E, 2 ff, W] stacks every
+    expert's gate rows on its up rows; w_down [E, W, ff].  On the GPU: one planning kernel sorts
+    the (row, choice) pairs by expert into tiles of MOE_TILE_ROWS (or MOE_BIG_TILE_ROWS), then two
+    grouped matrix products (gate | up with the activation in the epilogue; down) run over the
+    tiles - no host synchronisation, so the step can be captured in a graph.  Steps whose expert
+    products reach MOE_LIBRARY_FLOPS run library products per expert instead (outside a capture)."""
+    if not h.is_cuda:
+        return mref.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha)
+    T, W = h.shape
+    E, ff = w_gu.shape[0], w_gu.shape[1] // 2
+    k = idx.shape[1]
+    P = T * k
+    if 0 < MOE_LIBRARY_FLOPS <= 6.0 * P * ff * W and not torch.cuda.is_current_stream_capturing():
+        return _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha)
+    big = (h.dtype == torch.bfloat16 and W % 8 == 0 and ff % 8 == 0 and P >= MOE_BIG_TILE_PAIRS)
+    rows = MOE_BIG_TILE_ROWS if big else MOE_TILE_ROWS
+    max_tiles = P // rows + min(E, P)
+    dev = h.device
+    # few tiles (a decode step): the down product's long K range is cut over `split` workgroups
+    # per tile so the launch fills the chip; the fp32 partials are summed with the row's choices
+    split = 1
+    groups = max_tiles * -(-W // MOE_TILE_ROWS)
+    if h.dtype == torch.bfloat16 and W % 8 == 0 and ff % 8 == 0 and not big and groups < 1024:
+        split = max(1, min(8, 2048 // groups, ff // 256))
+    plan = torch.empty(2 + 3 * max_tiles + P, dtype=torch.int32, device=dev)
+    act = torch.empty(P, ff, dtype=h.dtype, device=dev)
+    y = torch.empty(P * split, W, dtype=torch.float32 if split > 1 else h.dtype, device=dev)
+    _native().moe_experts(y, act, plan, h, idx, wts, w_gu[:, :ff], w_gu[:, ff:], w_down,
+                          float(limit), float(alpha), max_tiles, rows, split)
+    return _pair_sum(y, T, k * split, h.dtype)

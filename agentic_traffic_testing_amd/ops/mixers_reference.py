@@ -66,11 +66,14 @@ def rotate_interleaved(x, cos_sin):
 
 
 def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
-                       k_cache, v_cache, heads, kv_heads, dim, vdim):
-    """Per-head RMS norm (plain weight) and rotary positions on q [T, heads * dim] and
-    k [T, kv_heads * dim] (row-strided views); returns q [T, heads, dim] and writes k and
-    v [T, kv_heads * vdim] into the paged caches k_cache [nb, kv_heads, BS, dim],
-    v_cache [nb, kv_heads, vdim, BS] (channel-major pages)."""
+                       k_cache, v_cache, heads, kv_heads, dim, vdim, rotate_half_pairs=False,
+                       norm_last=False):
+    """Per-head RMS norm (plain weight, or none when ``q_norm`` / ``k_norm`` is None) and rotary
+    positions on q [T, heads * dim] and k [T, kv_heads * dim] (row-strided views); returns
+    q [T, heads, dim] and writes k and v [T, kv_heads * vdim] into the paged caches
+    k_cache [nb, kv_heads, BS, dim], v_cache [nb, kv_heads, vdim, BS] (channel-major pages).
+    ``rotate_half_pairs``: channel i pairs with i + n instead of (2i, 2i + 1); ``norm_last``: the
+    norm follows the rotation instead of preceding it."""
     T = qx.shape[0]
     dt = qx.dtype
     q = qx.reshape(T, heads, dim).float()
@@ -78,10 +81,14 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     v = vx.reshape(T, kv_heads, vdim)
 
     def nrm(x, w):
-        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        return y * w.float() if w is not None else y
 
-    q = rotate_interleaved(nrm(q, q_norm), cos_sin).to(dt)
-    k = rotate_interleaved(nrm(k, k_norm), cos_sin).to(dt)
+    rot = rotate_half if rotate_half_pairs else rotate_interleaved
+    if norm_last:
+        q, k = nrm(rot(q, cos_sin), q_norm).to(dt), nrm(rot(k, cos_sin), k_norm).to(dt)
+    else:
+        q, k = rot(nrm(q, q_norm), cos_sin).to(dt), rot(nrm(k, k_norm), cos_sin).to(dt)
     bs = k_cache.shape[2]
     sm = slot_mapping.long()
     ok = sm >= 0
@@ -93,10 +100,11 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
 
 
 def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, scale, sink,
-                   sink_values=None):
+                   sink_values=None, window=0):
     """Causal paged attention of every portion's rows over its sequence's cached keys; fp32
     scores and weights; ``sink`` adds exp(s - max) to each denominator, s = 0 or the head's
-    entry of ``sink_values`` [H].  q [T, H, d] -> [T, H, dv]."""
+    entry of ``sink_values`` [H]; ``window`` > 0: a row at position i sees keys j with
+    0 <= i - j < window.  q [T, H, d] -> [T, H, dv]."""
     T, H, _ = q.shape
     G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     out = torch.zeros(T, H, dv, dtype=q.dtype, device=q.device)
@@ -114,7 +122,10 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, sca
         n = b - a
         sc = torch.einsum("qhd,hkd->hqk", q[a:b].float(), k) * scale
         qpos = torch.arange(kvlen - n, kvlen, device=q.device)
-        mask = torch.arange(kvlen, device=q.device)[None, :] > qpos[:, None]
+        kpos = torch.arange(kvlen, device=q.device)
+        mask = kpos[None, :] > qpos[:, None]
+        if window > 0:
+            mask = mask | (kpos[None, :] <= qpos[:, None] - window)
         sc = sc.masked_fill(mask[None], float("-inf"))
         m = sc.amax(-1, keepdim=True)
         if sink:
@@ -219,8 +230,9 @@ def residual_add(x, a, sa, b=None, sb=1.0, c=None):
     return x
 
 
-def embed_scale(table, ids, scale):
-    return table[ids.long()].float() * scale
+def embed_scale(table, ids, scale, copies=0):
+    x = table[ids.long()].float() * scale
+    return x.unsqueeze(1).repeat(1, copies, 1) if copies else x
 
 
 def rms_norm_rows(x, w, eps):
@@ -325,3 +337,104 @@ def state_space_scan(x, B, C, dt, dt_bias, a_log, skip, state, positions, seq_qs
             out[t] = torch.einsum("hnv,hn->hv", S, Cf[t]) + skip.float()[:, None] * xx[t]
         state[slot] = S
     return out
+
+
+# ---- hyper-connections, token shift, minGRU, gates, GELU, expert routing -----------------------
+
+def hyper_norm(xs, w_in, w, eps, dtype):
+    """xs fp32 [T, s, W] residual streams: RMS norm (weight w) of u = sum_s w_in[s] xs[:, s]."""
+    u = (xs.float() * w_in.float()[None, :, None]).sum(1)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(dtype)
+
+
+def hyper_update(xs, y, mix, w_out):
+    """All streams at once from the old ones: xs[:, t] = sum_s mix[s, t] xs[:, s] + w_out[t] y."""
+    new = torch.einsum("tsw,sr->trw", xs.float(), mix.float()) + \
+        w_out.float()[None, :, None] * y.float()[:, None, :]
+    xs.copy_(new)
+    return xs
+
+
+def token_shift(n, mu, shift_state, positions, seq_qstart, seq_slot, dtype):
+    """h = n + (n_prev - n) * mu per channel, n_prev the previous token's row of n (zeros before
+    position 0, ``shift_state[slot]`` before a later portion's first row); the portion's last row
+    of n becomes the new ``shift_state[slot]``.  n fp32 [T, W] -> [T, W] of ``dtype``."""
+    out = torch.zeros(n.shape, dtype=dtype, device=n.device)
+    nf = n.float()
+    for s, slot, a, b in _portions(seq_qstart, seq_slot):
+        first = shift_state[slot].float().clone()
+        if int(positions[a]) == 0:
+            first.zero_()
+        prev = torch.cat([first[None], nf[a:b - 1]], 0)
+        out[a:b] = (nf[a:b] + (prev - nf[a:b]) * mu.float()).to(dtype)
+        shift_state[slot] = nf[b - 1]
+    return out
+
+
+def gate_mul(a, gate, act):
+    """a [T, N] times sigmoid (act 1) or SiLU (act 0) of gate [T, N] (row-strided)."""
+    g = gate.float()
+    g = torch.sigmoid(g) if act == 1 else g * torch.sigmoid(g)
+    return (a.float() * g).to(a.dtype)
+
+
+def mingru_scan(z, x, g, state, positions, seq_qstart, seq_slot, dtype):
+    """minGRU: gate sigmoid(z), candidate x + 1/2 (x >= 0) or sigmoid(x) (x < 0),
+    S = (1 - gate) S + gate * candidate per channel, output S * silu(g).  z, x, g [T, C]
+    (row-strided); state fp32 [slots, C] advanced in place; all of it in fp32."""
+    T, C = z.shape
+    gate = torch.sigmoid(z.float())
+    xf = x.float()
+    cand = torch.where(xf >= 0, xf + 0.5, torch.sigmoid(xf))
+    gf = g.float()
+    og = gf * torch.sigmoid(gf)
+    out = torch.zeros(T, C, dtype=dtype, device=z.device)
+    st = state.view(state.shape[0], C)
+    for s, slot, a, b in _portions(seq_qstart, seq_slot):
+        S = st[slot].clone()
+        if int(positions[a]) == 0:
+            S.zero_()
+        for t in range(a, b):
+            S = S + gate[t] * (cand[t] - S)
+            out[t] = (S * og[t]).to(dtype)
+        st[slot] = S
+    return out
+
+
+def gelu(x, tanh_form=False):
+    return F.gelu(x.float(), approximate="tanh" if tanh_form else "none").to(x.dtype)
+
+
+def moe_route(logits, top):
+    """Sigmoid scores of fp32 router logits [T, E]; the ``top`` largest per row (ties: lowest
+    index) -> (int32 [T, top], fp32 [T, top])."""
+    s = torch.sigmoid(logits.float())
+    order = torch.argsort(s, dim=1, descending=True, stable=True)[:, :top]
+    return order.to(torch.int32), torch.gather(s, 1, order)
+
+
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha):
+    """Sum over a row's chosen experts of W_down act(W_gate (w h), W_up (w h)) with
+    act(g, u) = g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit).
+    h [T, W]; idx / wts [T, k]; w_gu [E, 2 ff, W] (gate rows, then up rows); w_down [E, W, ff].
+    fp32 accumulation, the activation rounded to h's dtype between the two products like the
+    kernels do."""
+    T, W = h.shape
+    out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
+    hf = h.float()
+    for j in range(idx.shape[1]):
+        for e in torch.unique(idx[:, j]).tolist():
+            rows = (idx[:, j] == e).nonzero().flatten()
+            a = clamped_glu(hf[rows] @ w_gu[e].float().T, wts[rows, j], limit, alpha).to(h.dtype)
+            out[rows] += (a.float() @ w_down[e].float().T).to(h.dtype).float()
+    return out.to(h.dtype)
+
+
+def clamped_glu(gu, wts, limit, alpha):
+    """Rows of [gate | up] products [R, 2 ff] and their router weights [R] -> the clamped GLU
+    activation [R, ff] (see ``moe_experts``)."""
+    ff = gu.shape[1] // 2
+    w = wts.float()[:, None]
+    g = (gu[:, :ff].float() * w).clamp(max=limit)
+    u = (gu[:, ff:].float() * w).clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
