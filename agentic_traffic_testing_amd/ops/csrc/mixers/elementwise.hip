@@ -209,15 +209,20 @@ __global__ void gated_rms_norm_kernel(T* __restrict__ out, const float* __restri
 }
 
 
-// Token embedding times a constant into the fp32 residual stream; one block per row.
+// Token embedding times a constant into the fp32 residual stream, `copies` times per row (the
+// streams of a multi-stream residual all start as the embedding); one block per row.
 template <typename T>
 __global__ void embed_scale_kernel(float* __restrict__ out, const T* __restrict__ table,
-                                   const int* __restrict__ ids, int W, int vocab, float scale) {
+                                   const int* __restrict__ ids, int W, int vocab, float scale,
+                                   int copies) {
   const int id = ids[blockIdx.x];
-  float* o = out + static_cast<int64_t>(blockIdx.x) * W;
+  float* o = out + static_cast<int64_t>(blockIdx.x) * copies * W;
   const bool ok = id >= 0 && id < vocab;
   const T* e = table + static_cast<int64_t>(ok ? id : 0) * W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) o[i] = ok ? ldf(e + i) * scale : 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float v = ok ? ldf(e + i) * scale : 0.f;
+    for (int c = 0; c < copies; ++c) o[c * W + i] = v;
+  }
 }
 
 // RMS norm with a plain weight over rows of activations (row-strided input): one wave per row.
@@ -455,10 +460,11 @@ extern "C" int mixk_gated_rms_norm(void* out, const float* o, const void* gate,
 }
 
 extern "C" int mixk_embed_scale(float* out, const void* table, const int* ids, int T_, int W,
-                                int vocab, float scale, int dtype, hipStream_t st) {
+                                int vocab, float scale, int copies, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
   MIXK_DISPATCH(dtype, hipLaunchKernelGGL(embed_scale_kernel<T>, dim3(T_), dim3(256), 0, st, out,
-                                          static_cast<const T*>(table), ids, W, vocab, scale));
+                                          static_cast<const T*>(table), ids, W, vocab, scale,
+                                          copies));
   return static_cast<int>(hipGetLastError());
 }
 
