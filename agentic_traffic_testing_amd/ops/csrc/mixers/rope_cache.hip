@@ -1,5 +1,6 @@
-// Per-head q / k RMS norm (plain weight), interleaved-pair rotary positions on the first
-// 2 * n_freq channels, and the paged K / V write of the softmax mixer; further down, the front
+// Per-head q / k RMS norm (plain weight or none), rotary positions on the first 2 * n_freq
+// channels (pairs (2i, 2i + 1), or (i, i + n_freq) in the rotate-half layout; the norm before or
+// after the rotation), and the paged K / V write of the softmax mixer; further down, the front
 // end of latent attention (absorbed query assembly, rotate-half positions, latent K / V write).
 //
 // Grid (rows, (H + G) / 4), four waves per workgroup, one wave per (row, head): heads [0, H)
@@ -36,7 +37,8 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                                           const int* __restrict__ slot_mapping,
                                           const float* __restrict__ cos_sin, int n_freq,
                                           T* __restrict__ k_cache, T* __restrict__ v_cache, int H,
-                                          int G, int dim, int vdim, int block_size) {
+                                          int G, int dim, int vdim, int block_size, int half,
+                                          int norm_last) {
   const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (head >= H + G) return;
   const int slot = slot_mapping[t];
@@ -48,6 +50,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                 : k_cache + ((static_cast<int64_t>(slot / block_size) * G + (head - H)) *
                                  block_size + slot % block_size) * dim;
   const int pairs = dim >> 1;
+  const float* tab = cos_sin + static_cast<int64_t>(t) * 2 * n_freq;   // [cos | sin] of row t
   float u[kMaxPairs], v[kMaxPairs];
   float ss = 0.f;
 #pragma unroll
@@ -55,29 +58,37 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
     const int i = lane + j * kWave;
     u[j] = v[j] = 0.f;
     if (i < pairs) {
-      u[j] = ldf(src + 2 * i);
-      v[j] = ldf(src + 2 * i + 1);
+      // pair i: channels (2i, 2i + 1), or (i, i + n_freq) for the rotated ones of the half layout
+      const int ca = (half && i < n_freq) ? i : 2 * i, cb = (half && i < n_freq) ? i + n_freq : 2 * i + 1;
+      u[j] = ldf(src + ca);
+      v[j] = ldf(src + cb);
+      if (norm_last && i < n_freq) {
+        const float cs = tab[i], sn = tab[n_freq + i];
+        const float ra = u[j] * cs - v[j] * sn;
+        v[j] = v[j] * cs + u[j] * sn;
+        u[j] = ra;
+      }
       ss += u[j] * u[j] + v[j] * v[j];
     }
   }
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(dim) + eps);
-  const float* tab = cos_sin + static_cast<int64_t>(t) * 2 * n_freq;   // [cos | sin] of row t
 #pragma unroll
   for (int j = 0; j < kMaxPairs; ++j) {
     const int i = lane + j * kWave;
     if (i >= pairs) continue;
-    float a = u[j] * inv * ldf(w + 2 * i);
-    float b = v[j] * inv * ldf(w + 2 * i + 1);
-    if (i < n_freq) {
+    const int ca = (half && i < n_freq) ? i : 2 * i, cb = (half && i < n_freq) ? i + n_freq : 2 * i + 1;
+    float a = u[j] * inv * (w != nullptr ? ldf(w + ca) : 1.0f);
+    float b = v[j] * inv * (w != nullptr ? ldf(w + cb) : 1.0f);
+    if (!norm_last && i < n_freq) {
       const float cs = tab[i], sn = tab[n_freq + i];
       const float ra = a * cs - b * sn;
       const float rb = b * cs + a * sn;
       a = ra;
       b = rb;
     }
-    stf(dst + 2 * i, a);
-    stf(dst + 2 * i + 1, b);
+    stf(dst + ca, a);
+    stf(dst + cb, b);
   }
 }
 
@@ -190,7 +201,8 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                        float eps, const int* positions, const int* slot_mapping,
                                        const float* cos_sin, int n_freq, void* k_cache,
                                        void* v_cache, int T_, int H, int G, int dim, int vdim,
-                                       int block_size, int dtype, hipStream_t st) {
+                                       int block_size, int half, int norm_last, int dtype,
+                                       hipStream_t st) {
   if (T_ <= 0) return 0;
   if (dim > 2 * kWave * kMaxPairs || (dim & 1)) return -1;
   MIXK_DISPATCH(dtype,
@@ -205,7 +217,7 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                    static_cast<const T*>(q_norm), static_cast<const T*>(k_norm),
                                    eps, positions, slot_mapping, cos_sin, n_freq,
                                    static_cast<T*>(k_cache), static_cast<T*>(v_cache), H, G, dim,
-                                   vdim, block_size));
+                                   vdim, block_size, half, norm_last));
   return static_cast<int>(hipGetLastError());
 }
 

@@ -21,6 +21,11 @@
 //   8+4h..8+4h+3 for lane half h), and the V^T operand reads follow the same order.
 // * combine kernel for the decode partials.
 //
+// A sliding window (`window` > 0: the query at position i sees keys j with 0 <= i - j < window)
+// moves the first key tile of a workgroup up to the window's start and masks the tiles that
+// touch its edge; decode then runs only the partitions that overlap the window (partition
+// indices are relative to the first of them, for the partition kernel and the combine alike).
+//
 // The sink enters as the initial state of the online softmax: running max = the sink's score,
 // running sum 1, zero accumulator.  The sink's score is 0, or one learned number per query head
 // (`sink_val`, unscaled).
@@ -45,7 +50,13 @@ struct AttnArgs {
   const float* sink_val;  // [H] score of the sink per query head (nullptr: 0)
   int bt_width, H, G, dim, vdim, block_size, sink, KT, max_parts, bs_shift;
   float scale;
+  int window;   // 0: every earlier key
 };
+
+// first key a query at position qpos sees
+__device__ __forceinline__ int window_start(int qpos, int window) {
+  return window > 0 ? max(0, qpos - window + 1) : 0;
+}
 
 template <typename T, bool DECODE>
 __global__ void __launch_bounds__(256)
@@ -66,9 +77,12 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
     kvlen = a.seq_kvlen[s];
     h0 = g * rep + (blockIdx.y % hb) * kRows;
     nrows = min(kRows, (g + 1) * rep - h0);
-    kbeg = blockIdx.z * kPartTokens;
+    if (kvlen <= 0) return;
+    const int wstart = window_start(kvlen - 1, a.window);
+    kbeg = (wstart / kPartTokens + blockIdx.z) * kPartTokens;
     kend = min(kvlen, kbeg + kPartTokens);
-    if (kvlen <= 0 || kbeg >= kend) return;
+    kbeg = max(kbeg, wstart);
+    if (kbeg >= kend) return;
   } else {
     const int tile = blockIdx.x >> 2;
     s = a.tile_seq[tile];
@@ -80,7 +94,7 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
     kvlen = a.seq_kvlen[s];
     if (n <= 0 || kvlen <= 0 || qo >= n) return;
     nrows = min(kRows, n - qo);
-    kbeg = 0;
+    kbeg = window_start(kvlen - n + qo, a.window);
     kend = min(kvlen, kvlen - n + qo + nrows);
   }
   const int tid = threadIdx.x, r = tid >> 4, c = tid & 15;
@@ -101,6 +115,7 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
   }
   const bool row_ok = r < nrows;
   const int qpos = DECODE ? kvlen - 1 : kvlen - n + qo + r;
+  const int qlow = window_start(qpos, a.window);
   const bool use_sink = a.sink && !DECODE;   // decode: the combine kernel adds the sink once
   float m = kNegBig, l = 0.f;
   if (use_sink) {
@@ -145,7 +160,7 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
       if (row_ok)
         for (int d = 0; d < dim; ++d) dot += qr[d] * kr[d];
       const int tok = k0 + kk;
-      sc[j] = (row_ok && tok <= qpos && tok < kend) ? dot * a.scale : kNegBig;
+      sc[j] = (row_ok && tok <= qpos && tok >= qlow && tok < kend) ? dot * a.scale : kNegBig;
       tmax = fmaxf(tmax, sc[j]);
     }
 #pragma unroll
@@ -208,7 +223,8 @@ __global__ void sink_attention_combine_kernel(T* __restrict__ out, AttnArgs a) {
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int kvlen = a.seq_kvlen[s];
   if (kvlen <= 0) return;
-  const int np = min(kMaxParts, (kvlen + kPartTokens - 1) / kPartTokens);
+  const int np = min(kMaxParts, (kvlen + kPartTokens - 1) / kPartTokens -
+                                    window_start(kvlen - 1, a.window) / kPartTokens);
   const int vdim = a.vdim, ps = vdim + 2;
   const float* base = a.part + (static_cast<int64_t>(s) * a.H + h) * a.max_parts * ps;
   const float sink_score = a.sink_val != nullptr ? a.sink_val[h] : 0.f;
@@ -273,7 +289,6 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   const int cols_total = ntok * rep;
   const int col0 = DECODE ? 0 : blockIdx.z * 128;
   if (col0 >= cols_total) return;
-  const int kbeg = DECODE ? blockIdx.z * kPartTokens : 0;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r = lane & 31, h = lane >> 5;
   const int col = col0 + w * 32 + r;
@@ -283,11 +298,20 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   const int64_t qrow = row0 + qo + tok;
   const int qpos = kvlen - n + qo + tok;
   const int last_tok = (min(cols_total, col0 + 128) - 1) / rep;
-  const int kend = DECODE ? min(kvlen, kbeg + kPartTokens)
+  // first key tile: the window's start of the workgroup's earliest column, on a tile boundary
+  // (the V^T staging reads 8 keys at a time from 8-aligned slots)
+  const int wstart = window_start(kvlen - n + qo + col0 / rep, a.window);
+  const int part0 = DECODE ? (wstart / kPartTokens + blockIdx.z) * kPartTokens : 0;
+  const int kbeg = max(part0, wstart & ~(kKeys - 1));
+  const int kend = DECODE ? min(kvlen, part0 + kPartTokens)
                           : min(kvlen, kvlen - n + qo + last_tok + 1);
   if (kbeg >= kend) return;
   const bool wave_on = col0 + w * 32 < cols_total;   // wave-uniform
   const int qpos_first = kvlen - n + qo + (col0 + w * 32) / rep;   // the wave's earliest column
+  // the wave's latest column: keys at or below its window start are outside somebody's window
+  const int qpos_lastw = kvlen - n + qo + (min(cols_total, col0 + w * 32 + 32) - 1) / rep;
+  const int edge_lo = a.window > 0 ? qpos_lastw - a.window : -1;
+  const int qlow = window_start(qpos, a.window);
   const float scale2 = a.scale * 1.44269504088896341f;
   const bool use_sink = a.sink && !DECODE;           // decode: the combine kernel adds it once
   bf16x8 qf[ND];
@@ -388,11 +412,13 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
     // scores in log2 units (scale * log2 e folded into one multiply; the sink's score 0 stays 0);
     // only tiles that reach the wave's causal edge or the end of the keys are masked
     float tmax = kNegBig;
-    if (k0 + kKeys - 1 > qpos_first || k0 + kKeys > kend) {
+    // (a masked score is -inf, the running maximum starts at the finite kNegBig: a column whose
+    // window has not begun yet keeps weight exp2(-inf) = 0 on every key of the tile)
+    if (k0 + kKeys - 1 > qpos_first || k0 + kKeys > kend || k0 <= edge_lo) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
-        S[i] = (key <= qpos && key < kend) ? S[i] * scale2 : kNegBig;
+        S[i] = (key <= qpos && key >= qlow && key < kend) ? S[i] * scale2 : -INFINITY;
         tmax = fmaxf(tmax, S[i]);
       }
     } else {
@@ -408,7 +434,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      S[i] = __builtin_amdgcn_exp2f(S[i] - m_new);   // masked scores: exp2(-1e30) = 0
+      S[i] = __builtin_amdgcn_exp2f(S[i] - m_new);   // masked scores: exp2(-inf) = 0
       psum += S[i];
     }
     psum += __shfl_xor(psum, 32, kWave);
@@ -481,6 +507,12 @@ int opt_in_smem(K kernel, size_t smem, size_t* opted) {
   return 0;
 }
 
+// partitions a decode row can touch: all of its context, or the ones its window overlaps
+int decode_parts(int max_decode_kv, int window) {
+  const int all = (max_decode_kv + kPartTokens - 1) / kPartTokens;
+  return window > 0 ? min(all, (window + kPartTokens - 1) / kPartTokens + 1) : all;
+}
+
 template <typename T>
 int launch_rows(void* out, const void* q, const void* k_cache, const void* v_cache, AttnArgs a,
                 int num_tiles, int num_decode, int max_decode_kv, hipStream_t st) {
@@ -498,7 +530,7 @@ int launch_rows(void* out, const void* q, const void* k_cache, const void* v_cac
   }
   if (num_decode > 0) {
     if (int rc = opt_in_smem(sink_attention_rows_kernel<T, true>, smem, &opted_d)) return rc;
-    const int parts = (max_decode_kv + kPartTokens - 1) / kPartTokens;
+    const int parts = decode_parts(max_decode_kv, a.window);
     if (parts > a.max_parts || parts < 1) return -1;
     const int head_blocks = (a.H / a.G + kRows - 1) / kRows;
     hipLaunchKernelGGL((sink_attention_rows_kernel<T, true>),
@@ -541,14 +573,15 @@ extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache
                                    const int* tile_seq, const int* tile_qoff, int num_tiles,
                                    int num_decode, int max_decode_kv, float* part, int max_parts,
                                    int H, int G, int dim, int vdim, int block_size, float scale,
-                                   int sink, const float* sink_val, int use_mfma, int dtype,
-                                   hipStream_t st) {
+                                   int sink, const float* sink_val, int window, int use_mfma,
+                                   int dtype, hipStream_t st) {
   if (num_tiles <= 0 && num_decode <= 0) return 0;
   if (vdim > 16 * kMaxVPer || G <= 0 || H % G != 0) return -1;
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
   AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, sink ? sink_val : nullptr,
-             bt_width, H, G, dim, vdim, block_size, sink, 0, max_parts, bs_shift, scale};
+             bt_width, H, G, dim, vdim, block_size, sink, 0, max_parts, bs_shift, scale,
+             window > 0 ? window : 0};
   int rc = 0;
   if (use_mfma) {
     if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size < 8 ||
@@ -556,7 +589,7 @@ extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache
       return -1;
     // decode columns = the query heads of one KV head: they must fit one workgroup
     const int nd_mfma = (H / G <= 128) ? num_decode : 0;
-    const int parts = (max_decode_kv + kPartTokens - 1) / kPartTokens;
+    const int parts = decode_parts(max_decode_kv, a.window);
     if (nd_mfma > 0 && (parts > max_parts || parts < 1)) return -1;
     if (dim <= 64 && vdim <= 64)
       launch_mfma<4, 2>(out, q, k_cache, v_cache, a, num_tiles, nd_mfma, parts, st);
