@@ -151,9 +151,11 @@ void gated_rms_norm(at::Tensor out, const at::Tensor& o, const at::Tensor& gate,
 }
 
 void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor& kx,
-                        const at::Tensor& vx, const at::Tensor& q_norm, const at::Tensor& k_norm,
-                        double eps, const at::Tensor& positions, const at::Tensor& slot_mapping,
-                        const at::Tensor& cos_sin, at::Tensor k_cache, at::Tensor v_cache) {
+                        const at::Tensor& vx, const c10::optional<at::Tensor>& q_norm,
+                        const c10::optional<at::Tensor>& k_norm, double eps,
+                        const at::Tensor& positions, const at::Tensor& slot_mapping,
+                        const at::Tensor& cos_sin, at::Tensor k_cache, at::Tensor v_cache,
+                        bool rotate_half, bool norm_last) {
   TORCH_CHECK(q_out.dim() == 3 && q_out.is_contiguous() && k_cache.dim() == 4 &&
                   v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "qk_norm_rope_cache: q_out [T, H, d], caches [nb, G, BS, d]");
@@ -173,20 +175,23 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                   v_cache.size(1) == G && v_cache.size(3) == BS &&
                   v_cache.size(0) == k_cache.size(0) && positions.numel() >= T &&
                   slot_mapping.numel() >= T && 2 * n_freq <= dim &&
-                  q_norm.numel() == dim && k_norm.numel() == dim && q_norm.is_contiguous() &&
-                  k_norm.is_contiguous() && k_cache.scalar_type() == q_out.scalar_type() &&
-                  v_cache.scalar_type() == q_out.scalar_type() &&
-                  q_norm.scalar_type() == q_out.scalar_type() &&
-                  k_norm.scalar_type() == q_out.scalar_type(),
+                  k_cache.scalar_type() == q_out.scalar_type() &&
+                  v_cache.scalar_type() == q_out.scalar_type(),
               "qk_norm_rope_cache: shapes");
+  for (const auto* w : {&q_norm, &k_norm})
+    if (w->has_value())
+      TORCH_CHECK((*w)->is_cuda() && (*w)->numel() == dim && (*w)->is_contiguous() &&
+                      (*w)->scalar_type() == q_out.scalar_type(),
+                  "qk_norm_rope_cache: norm weights [dim]");
   const at::DeviceGuard g(qx.device());
   rc_ok(mixk_qk_norm_rope_cache(q_out.data_ptr(), qx.data_ptr(), qx.stride(0), kx.data_ptr(),
-                                kx.stride(0), vx.data_ptr(), vx.stride(0), q_norm.data_ptr(),
-                                k_norm.data_ptr(), static_cast<float>(eps),
+                                kx.stride(0), vx.data_ptr(), vx.stride(0),
+                                q_norm ? q_norm->data_ptr() : nullptr,
+                                k_norm ? k_norm->data_ptr() : nullptr, static_cast<float>(eps),
                                 positions.data_ptr<int>(), slot_mapping.data_ptr<int>(),
                                 cos_sin.data_ptr<float>(), n_freq, k_cache.data_ptr(),
-                                v_cache.data_ptr(), T, H, G, dim, vdim, BS, code(q_out),
-                                cur_stream()),
+                                v_cache.data_ptr(), T, H, G, dim, vdim, BS, rotate_half, norm_last,
+                                code(q_out), cur_stream()),
         "qk_norm_rope_cache");
 }
 
@@ -209,7 +214,7 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
                     const at::Tensor& tile_seq, const at::Tensor& tile_qoff, double scale,
                     bool sink, int64_t num_decode, int64_t max_decode_kv,
                     const c10::optional<at::Tensor>& part, bool use_mfma,
-                    const c10::optional<at::Tensor>& sink_val) {
+                    const c10::optional<at::Tensor>& sink_val, int64_t window) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && out.dim() == 3 &&
                   out.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
                   k_cache.is_contiguous() && v_cache.is_contiguous(),
@@ -236,8 +241,9 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
     TORCH_CHECK(part.has_value(), "sink_attention: decode rows need the partials workspace");
     f32c(*part, "part");
     TORCH_CHECK(part->dim() == 4 && part->size(0) >= num_decode && part->size(1) == H &&
-                    part->size(3) == vdim + 2 && max_decode_kv >= 1 &&
-                    part->size(2) * 128 >= max_decode_kv,
+                    part->size(3) == vdim + 2 && max_decode_kv >= 1 && window >= 0 &&
+                    (part->size(2) * 128 >= max_decode_kv ||
+                     (window > 0 && part->size(2) >= (window + 127) / 128 + 1)),
                 "sink_attention: partials [num_decode, H, parts, vdim + 2]");
     part_ptr = part->data_ptr<float>();
     max_parts = part->size(2);
@@ -259,8 +265,8 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
                             seq_kvlen.data_ptr<int>(), seq_qstart.data_ptr<int>(),
                             tile_seq.data_ptr<int>(), tile_qoff.data_ptr<int>(), tile_seq.numel(),
                             num_decode, max_decode_kv, part_ptr, max_parts, H, G, dim, vdim, BS,
-                            static_cast<float>(scale), sink, sink_ptr, use_mfma, code(q),
-                            cur_stream()),
+                            static_cast<float>(scale), sink, sink_ptr, static_cast<int>(window),
+                            use_mfma, code(q), cur_stream()),
         "sink_attention");
 }
 
@@ -329,13 +335,15 @@ void gated_delta_rule(at::Tensor out, const at::Tensor& qkv, const at::Tensor& b
 void embed_scale(at::Tensor out, const at::Tensor& table, const at::Tensor& ids, double scale) {
   i32(ids, "ids");
   f32c(out, "out");
-  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous() && out.dim() == 2 &&
-                  out.size(0) == ids.numel() && out.size(1) == table.size(1),
+  // out [T, W], or [T, copies, W]: the row written `copies` times
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous() &&
+                  (out.dim() == 2 || out.dim() == 3) && out.size(0) == ids.numel() &&
+                  out.size(out.dim() - 1) == table.size(1),
               "embed_scale: shapes");
   const at::DeviceGuard g(table.device());
   rc_ok(mixk_embed_scale(out.data_ptr<float>(), table.data_ptr(), ids.data_ptr<int>(),
                          ids.numel(), table.size(1), table.size(0), static_cast<float>(scale),
-                         code(table), cur_stream()),
+                         out.dim() == 3 ? out.size(1) : 1, code(table), cur_stream()),
         "embed_scale");
 }
 
@@ -503,6 +511,182 @@ void gated_linear_scan(at::Tensor out, at::Tensor state, const at::Tensor& q, co
         "gated_linear_scan");
 }
 
+void hyper_update_norm(const c10::optional<at::Tensor>& out, at::Tensor xs,
+                       const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& mix,
+                       const c10::optional<at::Tensor>& w_out,
+                       const c10::optional<at::Tensor>& w_in, const c10::optional<at::Tensor>& w,
+                       double eps) {
+  f32c(xs, "xs");
+  TORCH_CHECK(xs.dim() == 3 && xs.size(1) >= 1 && xs.size(1) <= 8, "hyper_update_norm: xs [T, s, W]");
+  const int64_t T = xs.size(0), ns = xs.size(1), W = xs.size(2);
+  TORCH_CHECK(y.has_value() || w.has_value(), "hyper_update_norm: nothing to do");
+  int dt = -1;
+  if (y) {
+    TORCH_CHECK(y->is_cuda() && y->is_contiguous() && y->dim() == 2 && y->size(0) == T &&
+                    y->size(1) == W && mix.has_value() && w_out.has_value(),
+                "hyper_update_norm: y [T, W] with mix and w_out");
+    f32c(*mix, "mix");
+    f32c(*w_out, "w_out");
+    TORCH_CHECK(mix->numel() == ns * ns && w_out->numel() == ns, "hyper_update_norm: mix [s, s]");
+    dt = code(*y);
+  }
+  if (w) {
+    TORCH_CHECK(out.has_value() && w_in.has_value(), "hyper_update_norm: norm needs out and w_in");
+    f32c(*w_in, "w_in");
+    TORCH_CHECK(w->is_cuda() && w->is_contiguous() && w->numel() == W && w_in->numel() == ns &&
+                    out->is_cuda() && out->is_contiguous() && out->dim() == 2 &&
+                    out->size(0) == T && out->size(1) == W && (dt < 0 || dt == code(*w)) &&
+                    (out->scalar_type() == at::kFloat || out->scalar_type() == w->scalar_type()),
+                "hyper_update_norm: out [T, W] fp32 or of the weight's dtype");
+    dt = code(*w);
+  }
+  const at::DeviceGuard g(xs.device());
+  rc_ok(mixk_hyper_update_norm(w ? out->data_ptr() : nullptr,
+                               w && out->scalar_type() == at::kFloat, xs.data_ptr<float>(),
+                               y ? y->data_ptr() : nullptr, y ? mix->data_ptr<float>() : nullptr,
+                               y ? w_out->data_ptr<float>() : nullptr,
+                               w ? w_in->data_ptr<float>() : nullptr, w ? w->data_ptr() : nullptr,
+                               T, ns, W, static_cast<float>(eps), dt, cur_stream()),
+        "hyper_update_norm");
+}
+
+void token_shift(at::Tensor out, const at::Tensor& n, const at::Tensor& mu, at::Tensor state,
+                 const at::Tensor& positions, const at::Tensor& seq_qstart,
+                 const at::Tensor& seq_slot) {
+  f32c(n, "n");
+  f32c(mu, "mu");
+  f32c(state, "state");
+  TORCH_CHECK(n.dim() == 2, "token_shift: n [T, W]");
+  const int64_t T = n.size(0), W = n.size(1);
+  meta(positions, seq_qstart, seq_slot, T);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.sizes() == n.sizes() &&
+                  mu.numel() == W && state.dim() == 2 && state.size(1) == W,
+              "token_shift: shapes");
+  const at::DeviceGuard g(n.device());
+  rc_ok(mixk_token_shift(out.data_ptr(), n.data_ptr<float>(), mu.data_ptr<float>(),
+                         state.data_ptr<float>(), positions.data_ptr<int>(),
+                         seq_qstart.data_ptr<int>(), seq_slot.data_ptr<int>(), T, seq_slot.numel(),
+                         W, code(out), cur_stream()),
+        "token_shift");
+}
+
+void gate_mul(at::Tensor out, const at::Tensor& a, const at::Tensor& gate, int64_t act) {
+  rows2d(gate, out, "gate");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && a.is_cuda() && a.is_contiguous() &&
+                  a.dim() == 2 && out.sizes() == a.sizes() && gate.sizes() == a.sizes() &&
+                  a.scalar_type() == out.scalar_type(),
+              "gate_mul: shapes");
+  const at::DeviceGuard g(a.device());
+  rc_ok(mixk_gate_mul(out.data_ptr(), a.data_ptr(), gate.data_ptr(), gate.stride(0), a.size(0),
+                      a.size(1), act, code(out), cur_stream()),
+        "gate_mul");
+}
+
+void gelu(at::Tensor out, const at::Tensor& x, bool tanh_form) {
+  rows2d(x, out, "x");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes(), "gelu: out");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_gelu(out.data_ptr(), x.data_ptr(), x.stride(0), x.size(0), x.size(1), tanh_form,
+                  code(x), cur_stream()),
+        "gelu");
+}
+
+void mingru_scan(at::Tensor out, at::Tensor state, const at::Tensor& z, const at::Tensor& x,
+                 const at::Tensor& gt, const at::Tensor& positions, const at::Tensor& seq_qstart,
+                 const at::Tensor& seq_slot) {
+  rows2d(z, out, "z");
+  rows2d(x, out, "x");
+  rows2d(gt, out, "g");
+  f32c(state, "state");
+  const int64_t T = z.size(0), C = z.size(1), S = seq_slot.numel();
+  meta(positions, seq_qstart, seq_slot, T);
+  TORCH_CHECK(out.is_contiguous() && out.size(0) == T && out.size(1) == C && x.sizes() == z.sizes() &&
+                  gt.sizes() == z.sizes() && state.dim() >= 2 && state.numel() == state.size(0) * C,
+              "mingru_scan: shapes");
+  const at::DeviceGuard g(z.device());
+  rc_ok(mixk_mingru_scan(out.data_ptr(), state.data_ptr<float>(), z.data_ptr(), z.stride(0),
+                         x.data_ptr(), x.stride(0), gt.data_ptr(), gt.stride(0),
+                         positions.data_ptr<int>(), seq_qstart.data_ptr<int>(),
+                         seq_slot.data_ptr<int>(), S, C, T <= 4 * S, code(out), cur_stream()),
+        "mingru_scan");
+}
+
+void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits) {
+  f32c(logits, "logits");
+  f32c(wts, "wts");
+  i32(idx, "idx");
+  TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2 && idx.size(0) == logits.size(0) &&
+                  wts.sizes() == idx.sizes() && idx.size(1) >= 1 && idx.size(1) <= logits.size(1),
+              "moe_route: logits [T, E], idx / wts [T, top]");
+  const at::DeviceGuard g(logits.device());
+  rc_ok(mixk_moe_route(idx.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(),
+                       logits.size(0), logits.size(1), idx.size(1), cur_stream()),
+        "moe_route");
+}
+
+void moe_experts(at::Tensor y, at::Tensor act, at::Tensor plan, const at::Tensor& h,
+                 const at::Tensor& idx, const at::Tensor& wts, const at::Tensor& w_gate,
+                 const at::Tensor& w_up, const at::Tensor& w_down, double limit, double alpha,
+                 int64_t max_tiles, int64_t tile_rows, int64_t split) {
+  i32(idx, "idx");
+  i32(plan, "plan");
+  f32c(wts, "wts");
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous() && idx.dim() == 2 &&
+                  idx.size(0) == h.size(0) && wts.sizes() == idx.sizes() && w_gate.dim() == 3 &&
+                  w_down.is_contiguous() && w_up.sizes() == w_gate.sizes() && w_down.dim() == 3 &&
+                  w_gate.stride(2) == 1 && w_gate.stride(1) == w_gate.size(2) &&
+                  w_up.strides() == w_gate.strides() && w_gate.stride(0) % 8 == 0,
+              "moe_experts: h [T, W], idx / wts [T, top], w_gate / w_up [E, ff, W]");
+  const int64_t T = h.size(0), W = h.size(1), top = idx.size(1), E = w_gate.size(0);
+  const int64_t ff = w_gate.size(1), P = T * top;
+  TORCH_CHECK(w_gate.size(2) == W && w_down.size(0) == E && w_down.size(1) == W &&
+                  w_down.size(2) == ff && y.is_contiguous() && y.dim() == 2 && split >= 1 &&
+                  split <= 64 && y.size(0) == P * split && y.size(1) == W && act.is_contiguous() && act.dim() == 2 && act.size(0) == P &&
+                  act.size(1) == ff && plan.numel() >= 2 + 3 * max_tiles + P &&
+                  (tile_rows == 64 || tile_rows == 128) &&
+                  max_tiles >= P / tile_rows + std::min(E, P) && P < (int64_t{1} << 30) &&
+                  w_gate.scalar_type() == h.scalar_type() && w_up.scalar_type() == h.scalar_type() &&
+                  w_down.scalar_type() == h.scalar_type() &&
+                  y.scalar_type() == (split > 1 ? at::kFloat : h.scalar_type()) &&
+                  act.scalar_type() == h.scalar_type(),
+              "moe_experts: shapes");
+  const at::DeviceGuard g(h.device());
+  rc_ok(mixk_moe_experts(y.data_ptr(), act.data_ptr(), plan.data_ptr<int>(), h.data_ptr(),
+                         idx.data_ptr<int>(), wts.data_ptr<float>(), w_gate.data_ptr(),
+                         w_up.data_ptr(), w_down.data_ptr(), T, top, E, ff, W, w_gate.stride(0), max_tiles,
+                         tile_rows, split,
+                         static_cast<float>(limit), static_cast<float>(alpha), code(h),
+                         cur_stream()),
+        "moe_experts");
+}
+
+void pair_sum(at::Tensor out, const at::Tensor& y) {
+  TORCH_CHECK(y.is_cuda() && y.dim() == 3 && y.is_contiguous() && out.is_cuda() &&
+                  out.is_contiguous() && out.dim() == 2 && out.size(0) == y.size(0) &&
+                  out.size(1) == y.size(2) &&
+                  (out.scalar_type() == y.scalar_type() || y.scalar_type() == at::kFloat),
+              "pair_sum: y [T, top, W] (out's dtype or fp32), out [T, W]");
+  const at::DeviceGuard g(y.device());
+  rc_ok(mixk_pair_sum(out.data_ptr(), y.data_ptr(), y.scalar_type() == at::kFloat, y.size(0),
+                      y.size(1), y.size(2), code(out), cur_stream()),
+        "pair_sum");
+}
+
+void clamped_glu(at::Tensor out, const at::Tensor& gu, const at::Tensor& wts, double limit,
+                 double alpha) {
+  f32c(wts, "wts");
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.is_contiguous() && gu.size(1) % 2 == 0 &&
+                  out.is_cuda() && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == gu.size(0) && out.size(1) * 2 == gu.size(1) &&
+                  wts.numel() == gu.size(0) && out.scalar_type() == gu.scalar_type(),
+              "clamped_glu: gu [R, 2 ff], out [R, ff], wts [R]");
+  const at::DeviceGuard g(gu.device());
+  rc_ok(mixk_clamped_glu(out.data_ptr(), gu.data_ptr(), wts.data_ptr<float>(), gu.size(0),
+                         out.size(1), static_cast<float>(limit), static_cast<float>(alpha),
+                         code(gu), cur_stream()),
+        "clamped_glu");
+}
+
 }  // namespace
 
 TORCH_LIBRARY(atta_mix, m) {
@@ -515,14 +699,14 @@ TORCH_LIBRARY(atta_mix, m) {
   m.def("add_norm(Tensor(a!) h, Tensor(b!) x, Tensor a, float sa, Tensor? b, float sb, Tensor? c, "
         "Tensor w, float eps, bool one_plus) -> ()");
   m.def("gated_rms_norm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, float eps, int act) -> ()");
-  m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor q_norm, "
-        "Tensor k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor cos_sin, "
-        "Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
+  m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor? q_norm, "
+        "Tensor? k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor cos_sin, "
+        "Tensor(b!) k_cache, Tensor(c!) v_cache, bool rotate_half, bool norm_last) -> ()");
   m.def("rotary_table(Tensor(a!) out, Tensor positions, Tensor inv_freq) -> ()");
   m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
         "Tensor tile_qoff, float scale, bool sink, int num_decode, int max_decode_kv, "
-        "Tensor? part, bool use_mfma, Tensor? sink_val) -> ()");
+        "Tensor? part, bool use_mfma, Tensor? sink_val, int window) -> ()");
   m.def("short_conv_silu(Tensor(a!) out, Tensor x, Tensor w, Tensor(b!) conv_state, "
         "Tensor positions, Tensor seq_qstart, Tensor seq_slot, Tensor? bias) -> ()");
   m.def("gated_delta_rule(Tensor(a!) out, Tensor qkv, Tensor beta, Tensor decay, Tensor a_log, "
@@ -540,6 +724,20 @@ TORCH_LIBRARY(atta_mix, m) {
   m.def("gated_linear_scan(Tensor(a!) out, Tensor(b!) state, Tensor q, Tensor k, Tensor v, "
         "Tensor? dt, Tensor p0, Tensor p1, Tensor? p2, Tensor positions, Tensor seq_qstart, "
         "Tensor seq_slot, int H, int G, int dk, int dv, int mode) -> ()");
+  m.def("hyper_update_norm(Tensor(a!)? out, Tensor(b!) xs, Tensor? y, Tensor? mix, Tensor? w_out, "
+        "Tensor? w_in, Tensor? w, float eps) -> ()");
+  m.def("token_shift(Tensor(a!) out, Tensor n, Tensor mu, Tensor(b!) state, Tensor positions, "
+        "Tensor seq_qstart, Tensor seq_slot) -> ()");
+  m.def("gate_mul(Tensor(a!) out, Tensor a, Tensor gate, int act) -> ()");
+  m.def("gelu(Tensor(a!) out, Tensor x, bool tanh_form) -> ()");
+  m.def("mingru_scan(Tensor(a!) out, Tensor(b!) state, Tensor z, Tensor x, Tensor g, "
+        "Tensor positions, Tensor seq_qstart, Tensor seq_slot) -> ()");
+  m.def("pair_sum(Tensor(a!) out, Tensor y) -> ()");
+  m.def("clamped_glu(Tensor(a!) out, Tensor gu, Tensor wts, float limit, float alpha) -> ()");
+  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits) -> ()");
+  m.def("moe_experts(Tensor(a!) y, Tensor(b!) act, Tensor(c!) plan, Tensor h, Tensor idx, "
+        "Tensor wts, Tensor w_gate, Tensor w_up, Tensor w_down, float limit, float alpha, "
+        "int max_tiles, int tile_rows, int split) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
@@ -561,4 +759,13 @@ TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
   m.impl("head_gate", &head_gate);
   m.impl("latent_rope_cache", &latent_rope_cache);
   m.impl("gated_linear_scan", &gated_linear_scan);
+  m.impl("hyper_update_norm", &hyper_update_norm);
+  m.impl("token_shift", &token_shift);
+  m.impl("gate_mul", &gate_mul);
+  m.impl("gelu", &gelu);
+  m.impl("mingru_scan", &mingru_scan);
+  m.impl("pair_sum", &pair_sum);
+  m.impl("clamped_glu", &clamped_glu);
+  m.impl("moe_route", &moe_route);
+  m.impl("moe_experts", &moe_experts);
 }

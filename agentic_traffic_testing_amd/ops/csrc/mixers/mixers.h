@@ -26,7 +26,7 @@ int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_stride, const
                             const void* k_norm, float eps, const int* positions,
                             const int* slot_mapping, const float* cos_sin, int n_freq,
                             void* k_cache, void* v_cache, int T, int H, int G, int dim, int vdim,
-                            int block_size, int dtype, hipStream_t st);
+                            int block_size, int half, int norm_last, int dtype, hipStream_t st);
 int mixk_rotary_table(float* out, const int* positions, const float* inv_freq, int T, int n_freq,
                       hipStream_t st);
 int mixk_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -34,8 +34,8 @@ int mixk_sink_attention(void* out, const void* q, const void* k_cache, const voi
                         const int* seq_qstart, const int* tile_seq, const int* tile_qoff,
                         int num_tiles, int num_decode, int max_decode_kv, float* part,
                         int max_parts, int H, int G, int dim, int vdim, int block_size,
-                        float scale, int sink, const float* sink_val, int use_mfma, int dtype,
-                        hipStream_t st);
+                        float scale, int sink, const float* sink_val, int window, int use_mfma,
+                        int dtype, hipStream_t st);
 int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
                          const void* bias, void* conv_state, const int* positions, const int* seq_qstart,
                          const int* seq_slot, int T, int S, int C, int taps, int dtype,
@@ -46,7 +46,7 @@ int mixk_gated_delta_rule(float* out, const void* qkv, const void* beta, int64_t
                           const int* positions, const int* seq_qstart, const int* seq_slot, int S,
                           int H, int G, int dim, int vdim, int dtype, hipStream_t st);
 int mixk_embed_scale(float* out, const void* table, const int* ids, int T, int W, int vocab,
-                     float scale, int dtype, hipStream_t st);
+                     float scale, int copies, int dtype, hipStream_t st);
 int mixk_rms_norm_rows(void* out, const void* x, int64_t x_stride, const void* w, int T, int N,
                        float eps, int dtype, hipStream_t st);
 int mixk_xielu_bias(void* out, const void* x, int64_t x_stride, const void* bias, int T, int N,
@@ -67,4 +67,29 @@ int mixk_gated_linear_scan(float* out, float* state, const void* q, int64_t q_st
                            const float* p2, const int* positions, const int* seq_qstart,
                            const int* seq_slot, int S, int H, int G, int dk, int dv, int mode,
                            int dtype, hipStream_t st);
+int mixk_hyper_update_norm(void* out, int out_f32, float* xs, const void* y, const float* mix,
+                           const float* w_out, const float* w_in, const void* w, int T, int ns,
+                           int W, float eps, int dtype, hipStream_t st);
+int mixk_token_shift(void* out, const float* n, const float* mu, float* state,
+                     const int* positions, const int* seq_qstart, const int* seq_slot, int T,
+                     int S, int W, int dtype, hipStream_t st);
+int mixk_gate_mul(void* out, const void* a, const void* gate, int64_t gate_stride, int T, int N,
+                  int act, int dtype, hipStream_t st);
+int mixk_gelu(void* out, const void* x, int64_t x_stride, int T, int N, int tanh_form, int dtype,
+              hipStream_t st);
+int mixk_mingru_scan(void* out, float* state, const void* z, int64_t z_stride, const void* x,
+                     int64_t x_stride, const void* g, int64_t g_stride, const int* positions,
+                     const int* seq_qstart, const int* seq_slot, int S, int C, int few_rows,
+                     int dtype, hipStream_t st);
+int mixk_clamped_glu(void* out, const void* gu, const float* wts, int R, int ff, float limit,
+                     float alpha, int dtype, hipStream_t st);
+int mixk_pair_sum(void* out, const void* y, int y_f32, int T, int top, int W, int dtype,
+                  hipStream_t st);
+int mixk_moe_route(int* idx, float* wts, const float* logits, int T, int E, int top,
+                   hipStream_t st);
+int mixk_moe_experts(void* y, void* act, int* plan, const void* h, const int* idx,
+                     const float* wts, const void* w_gate, const void* w_up, const void* w_down,
+                     int T, int top, int E, int ff, int W, int64_t gu_estride, int max_tiles,
+                     int tile_rows, int split, float limit,
+                     float alpha, int dtype, hipStream_t st);
 }
