@@ -386,3 +386,191 @@ def test_biased_conv_gated_group_norm_xielu_head_gate(dt):
     wr = (1 + 0.1 * torch.randn(128)).to(dt)
     assert torch.allclose(mx.rms_norm_rows(x.cuda()[:, 8:], wr.cuda(), 1e-6).cpu().float(),
                           mref.rms_norm_rows(x[:, 8:], wr, 1e-6).float(), **tol(dt))
+
+
+# ---- multi-stream residual, token shift, window attention, minGRU, routed experts ------------
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("ns,W", [(2, 96), (3, 1024), (1, 100), (4, 4096), (2, 20000)])
+def test_hyper_update_norm(dt, ns, W):
+    torch.manual_seed(11)
+    T = 9
+    xs = torch.randn(T, ns, W) * 2
+    y = torch.randn(T, W).to(dt)
+    mix, w_out, w_in = torch.randn(ns, ns), torch.randn(ns), torch.randn(ns)
+    w = (1 + 0.1 * torch.randn(W)).to(dt)
+    for out_dt in (dt, torch.float32):
+        xr, xg = xs.clone(), xs.clone().cuda()
+        want = mref.hyper_norm(mref.hyper_update(xr, y, mix, w_out), w_in, w, 1e-6, out_dt)
+        got = mx.hyper_update_norm(xg, y.cuda(), mix.cuda(), w_out.cuda(), w_in.cuda(), w.cuda(),
+                                   1e-6, out_dt)
+        assert got.dtype == out_dt
+        assert torch.allclose(xg.cpu(), xr, atol=1e-4, rtol=1e-5)
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(out_dt if out_dt == dt else
+                                                                     torch.float32))
+        # norm only / update only
+        a = mx.hyper_norm(xg, w_in.cuda(), w.cuda(), 1e-6, out_dt)
+        assert torch.allclose(a.cpu().float(), want.float(), **tol(dt))
+    x2 = xs.clone().cuda()
+    assert mx.hyper_update_norm(x2, y.cuda(), mix.cuda(), w_out.cuda(), None, None, 1e-6) is None
+    assert torch.allclose(x2.cpu(), mref.hyper_update(xs.clone(), y, mix, w_out), atol=1e-4,
+                          rtol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_token_shift_gate_gelu(dt):
+    torch.manual_seed(12)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, W = int(md["seq_qstart"][-1]), 72
+    n, mu = torch.randn(T, W), torch.rand(W)
+    st = torch.randn(5, W)
+    st_g = st.clone().cuda()
+    want = mref.token_shift(n, mu, st, md["positions"], md["seq_qstart"], md["seq_slot"], dt)
+    got = mx.token_shift(n.cuda(), mu.cuda(), st_g, mdg["positions"], mdg["seq_qstart"],
+                         mdg["seq_slot"], dt)
+    rows = live_rows(md, LENS, SLOTS)
+    assert torch.allclose(got.cpu().float()[rows], want.float()[rows], **tol(dt))
+    assert torch.equal(st_g.cpu(), st)
+    for N, off in ((96, 8), (50, 3)):
+        big = torch.randn(T, 2 * N + 16).to(dt)
+        a = torch.randn(T, N).to(dt)
+        for act in ("sigmoid", "silu"):
+            assert torch.allclose(mx.gate_mul(a.cuda(), big.cuda()[:, off:off + N], act).cpu().float(),
+                                  mx.gate_mul(a, big[:, off:off + N], act).float(), **tol(dt))
+        for tanh_form in (False, True):
+            assert torch.allclose(mx.gelu(big.cuda()[:, off:off + N], tanh_form).cpu().float(),
+                                  mref.gelu(big[:, off:off + N], tanh_form).float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,rot", [(6, 2, 64, 24), (4, 1, 48, 48), (8, 2, 128, 64), (2, 2, 32, 0)])
+def test_rotate_half_norm_last_front_end(dt, H, G, dim, rot):
+    """Rotate-half pairs, rotation before a weightless norm, values = the raw key projection."""
+    torch.manual_seed(13)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, nb, bs = int(md["seq_qstart"][-1]), md["num_pages"], 16
+    P = torch.randn(T, (H + G) * dim + 16).to(dt)
+    sl = (slice(None), slice(8, 8 + H * dim)), (slice(None), slice(8 + H * dim, 8 + (H + G) * dim))
+    inv = mx.scaled_inv_freq(rot, 30000.0, (3.0, 1.0, 5.0, 256.0), "cpu")
+    tab = mref.rotary_table(md["positions"], inv)
+    kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, dim, bs).to(dt)
+    kcg, vcg, Pg = kc.cuda(), vc.cuda(), P.cuda()
+    qr = mref.qk_norm_rope_cache(P[sl[0]], P[sl[1]], P[sl[1]], None, None, 1e-6, md["positions"],
+                                 md["slot_mapping"], tab, kc, vc, H, G, dim, dim, True, True)
+    qg = mx.qk_norm_rope_cache(Pg[sl[0]], Pg[sl[1]], Pg[sl[1]], None, None, 1e-6,
+                               mdg["positions"], mdg["slot_mapping"], tab.cuda(), kcg, vcg, H, G,
+                               dim, dim, True, True)
+    assert torch.allclose(qg.cpu().float(), qr.float(), **tol(dt))
+    assert torch.allclose(kcg.cpu().float(), kc.float(), **tol(dt))
+    assert torch.equal(vcg.cpu(), vc)
+
+
+def test_scaled_inv_freq_bands():
+    f = mx.inv_freq(32, 10000.0, "cpu").double()
+    g = mx.scaled_inv_freq(32, 10000.0, (8.0, 1.0, 4.0, 64.0), "cpu").double()
+    wave = 2 * np.pi / f
+    for i in range(16):
+        if wave[i] < 16:
+            assert abs(g[i] - f[i]) < 1e-7 * f[i]
+        elif wave[i] > 64:
+            assert abs(g[i] - f[i] / 8) < 1e-7 * f[i]
+        else:
+            assert f[i] / 8 < g[i] < f[i]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,vdim", [(6, 2, 64, 64), (4, 1, 48, 80), (8, 2, 128, 128)])
+@pytest.mark.parametrize("window", [1, 31, 80, 128, 300])
+def test_window_attention(dt, H, G, dim, vdim, window):
+    """Windows shorter and longer than a tile, a partition and the contexts; decode rows whose
+    window starts inside, at the edge of and before their first partition."""
+    torch.manual_seed(14)
+    lens, starts = [1, 1, 1, 1, 150, 70, 2], [0, 127, 128, 700, 333, 0, 71]
+    md = ragged(lens, starts, list(range(7)), width=64)
+    keep = md["tile_seq"] >= 4
+    md["tile_seq"], md["tile_qoff"] = md["tile_seq"][keep], md["tile_qoff"][keep]
+    mdg = cuda(md)
+    T, nb = int(md["seq_qstart"][-1]), md["num_pages"]
+    q = torch.randn(T, H, dim).to(dt)
+    kc, vc = torch.randn(nb, G, 16, dim).to(dt), torch.randn(nb, G, vdim, 16).to(dt)
+    want = mref.sink_attention(q, kc, vc, md["block_tables"], md["seq_kvlen"], md["seq_qstart"],
+                               0.15, False, None, window)
+    for mfma in (True, False):
+        mx.ATTENTION_MFMA = mfma
+        try:
+            got = mx.sink_attention(q.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                    mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                    mdg["tile_qoff"], 0.15, False, num_decode=4, max_decode_kv=701,
+                                    window=window)
+        finally:
+            mx.ATTENTION_MFMA = True
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt)), (mfma, window)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("C", [200, 64, 100, 1024])
+def test_mingru_scan(dt, C):
+    torch.manual_seed(15)
+    lens, starts, slots = [1, 1, 37, 2, 600, 17], [0, 70, 0, 31, 5, 3], [3, -1, 0, 2, 1, 4]
+    md = ragged(lens, starts, slots, width=64)
+    mdg = cuda(md)
+    T = int(md["seq_qstart"][-1])
+    P = torch.randn(T, 3 * C + 24).to(dt) * 2
+    cut = lambda t: (t[:, 8:8 + C], t[:, 8 + C:8 + 2 * C], t[:, 16 + 2 * C:16 + 3 * C])  # noqa: E731
+    st = torch.randn(6, 1, 1, C)
+    st_g = st.clone().cuda()
+    want = mref.mingru_scan(*cut(P), st, md["positions"], md["seq_qstart"], md["seq_slot"], dt)
+    got = mx.mingru_scan(*cut(P.cuda()), st_g, mdg["positions"], mdg["seq_qstart"],
+                         mdg["seq_slot"], dt)
+    rows = live_rows(md, lens, slots)
+    assert torch.allclose(got.cpu().float()[rows], want.float()[rows], **tol(dt))
+    assert torch.allclose(st_g.cpu(), st, atol=1e-4, rtol=1e-4)
+    # a decode-sized step takes the one-wave path
+    md1 = ragged([1, 1, 1], [5, 0, 9], [2, 0, -1])
+    P1 = torch.randn(3, 3 * C + 24).to(dt)
+    st1 = st.clone()
+    st1_g = st.clone().cuda()
+    want = mref.mingru_scan(*cut(P1), st1, md1["positions"], md1["seq_qstart"], md1["seq_slot"], dt)
+    m1 = cuda(md1)
+    got = mx.mingru_scan(*cut(P1.cuda()), st1_g, m1["positions"], m1["seq_qstart"], m1["seq_slot"],
+                         dt)
+    assert torch.allclose(got.cpu().float()[:2], want.float()[:2], **tol(dt))
+    assert torch.allclose(st1_g.cpu(), st1, atol=1e-5)
+
+
+@pytest.mark.parametrize("E,top", [(10, 1), (6, 2), (70, 4), (3, 3)])
+def test_moe_route(E, top):
+    torch.manual_seed(16)
+    logits = torch.randn(200, E) * 3
+    logits[5, :] = 0.0              # all equal: the lowest indices win
+    idx, wts = mx.moe_route(logits.cuda(), top)
+    ri, rw = mref.moe_route(logits, top)
+    assert torch.equal(idx.cpu(), ri)
+    assert torch.allclose(wts.cpu(), rw, atol=1e-6)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("T,E,top,ff,W", [(150, 10, 1, 72, 328), (3, 6, 2, 48, 96), (700, 4, 2, 200, 136),
+                                          (65, 5, 3, 30, 50), (1, 8, 1, 128, 256), (5, 6, 2, 1024, 128),
+                                          (2, 3, 1, 584, 64)])
+def test_moe_experts(dt, T, E, top, ff, W):
+    """Matrix-core kernels (bf16, widths % 8 == 0; small and large tiles) and the rows kernels
+    (fp32, odd widths); tiles of one row and full tiles; clamps on both sides active; few tiles
+    with a long down product (its K range cut over several workgroups); the library path of
+    large steps against the grouped kernels."""
+    torch.manual_seed(17)
+    h = torch.randn(T, W).to(dt)
+    wgu = (torch.randn(E, 2 * ff, W) * 2 / W ** 0.5).to(dt)
+    wd = (torch.randn(E, W, ff) / ff ** 0.5).to(dt)
+    idx, wts = mref.moe_route(torch.randn(T, E) * 2, top)
+    want = mref.moe_experts(h, idx, wts, wgu, wd, 1.5, 1.702)
+    t = dict(atol=6e-2, rtol=3e-2) if dt == torch.bfloat16 else dict(atol=5e-5, rtol=5e-5)
+    for library_from in (0, 1):
+        old, mx.MOE_LIBRARY_FLOPS = mx.MOE_LIBRARY_FLOPS, library_from
+        try:
+            got = mx.moe_experts(h.cuda(), idx.cuda(), wts.cuda(), wgu.cuda(), wd.cuda(), 1.5, 1.702)
+        finally:
+            mx.MOE_LIBRARY_FLOPS = old
+        assert torch.allclose(got.cpu().float(), want.float(), **t), library_from

@@ -1,0 +1,636 @@
+"""Semezen through the serving engine (loader, paged window-attention cache, state slots for
+the minGRU state and the token-shift rows, scheduler, batching, sampling) and its mechanisms
+alone, against the slow oracle in tests/semezen_oracle.py.
+
+The engine runs on the CPU reference ops here and on the HIP kernels in the GPU tier (same
+tests, ``device`` parameter).  Configurations are small and irregular on purpose: three streams,
+windows that end inside pages, rotation on part of the head with and without frequency scaling,
+1 to all key / value heads, experts with top 1 / 2 / all, layers without feed-forward.
+"""
+import json
+import math
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import semezen_oracle as oracle
+from agentic_traffic_testing_amd.config import EngineConfig, SemezenConfig
+from agentic_traffic_testing_amd.engine.llm_engine import LLMEngine
+from agentic_traffic_testing_amd.engine.sequence import SamplingParams
+from agentic_traffic_testing_amd.models.semezen import SemezenModel
+from agentic_traffic_testing_amd.ops import mixers as mx
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+
+ATT = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 0.21, "mask": {"size": 21},
+       "rot": {"dims": 12, "base": 3000.0,
+               "scaling": {"factor": 6.0, "low": 1.0, "high": 3.0, "original": 40}}}
+GRU = {"width": 44}
+MOE = {"kind": "moe", "expert": {"ff": 24, "limit": 1.25}, "router": {"experts": 5, "top": 2}}
+
+
+def make_cfg(order="adgeae", width=48, vocab=97, streams=3, att=None, gru=None, moe=None, ff=40):
+    """Two letters per layer: mixer (a attention, g minGRU), feed-forward (d dense, e experts,
+    - none)."""
+    layers = []
+    for j in range(0, len(order), 2):
+        mlp = {"d": {"kind": "dense", "ff": ff}, "e": dict(moe or MOE), "-": None}[order[j + 1]]
+        if order[j] == "a":
+            layers.append({"type": "attention", "mixer": dict(att or ATT), "mlp": mlp})
+        else:
+            layers.append({"type": "mingru", "mixer": dict(gru or GRU), "mlp": mlp})
+    return {"architecture": "Semezen", "vocab": vocab, "width": width, "streams": streams,
+            "norm": {"eps": 3e-6}, "layers": layers}
+
+
+def make_params(cfg, seed=0):
+    shapes = SemezenModel(SemezenConfig.from_dict(cfg), torch.float32, "cpu").tensor_shapes()
+    g = torch.Generator().manual_seed(seed)
+    s = cfg["streams"]
+    p = {}
+    for name, shape in shapes.items():
+        r = torch.randn(shape, generator=g)
+        parts = name.split(".")
+        leaf = parts[-1]
+        if name == "embed":
+            t = r
+        elif leaf in ("norm1", "norm2", "norm"):
+            t = 1.1 + 0.3 * r
+        elif leaf == "shift":
+            t = torch.rand(shape, generator=g)
+        elif leaf == "b":
+            t = 0.5 * r
+        elif len(parts) > 1 and parts[1] in ("hc1", "hc2"):
+            t = {"in": 1.0 / s + 0.3 * r, "out": 0.8 + 0.3 * r}.get(leaf)
+            if t is None:
+                t = 0.7 * torch.eye(s) + 0.25 * r      # not symmetric: [from, to] matters
+        elif leaf == "router":
+            t = r * (6.0 / math.sqrt(shape[-1]))
+        else:
+            t = r * (1.5 / math.sqrt(shape[-1]))
+        p[name] = t.to(torch.bfloat16).contiguous()
+    return p
+
+
+@pytest.fixture(scope="module")
+def model_dir(tmp_path_factory):
+    made = {}
+
+    def get(key="default", **kw):
+        if key not in made:
+            d = tmp_path_factory.mktemp("semezen_" + key)
+            cfg = make_cfg(**kw)
+            params = make_params(cfg, seed=len(made))
+            (d / "config.json").write_text(json.dumps(cfg))
+            save_file(params, str(d / "model.safetensors"))
+            made[key] = (str(d), cfg, params)
+        return made[key]
+
+    return get
+
+
+def engine(path, device, dtype="float32", pool_tokens=512, max_seqs=4, block_size=16):
+    cfg = EngineConfig(model=path, device=device, dtype=dtype, block_size=block_size,
+                       max_model_len=pool_tokens, max_num_seqs=max_seqs,
+                       max_num_batched_tokens=max(512, pool_tokens),
+                       num_kv_blocks=pool_tokens // block_size, use_graphs=False,
+                       async_decode=False, startup_warmup=False, gemm_tuning="")
+    return LLMEngine(cfg)
+
+
+def close(got, want, dtype="float32"):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    err = np.sqrt((d ** 2).mean(-1)) / max(1e-9, float(np.sqrt((want ** 2).mean())))
+    if dtype != "float32":   # bf16 rounding: small on average, a few times that at single rows
+        assert err.mean() < 2e-2, f"mean relative logit error {err.mean():.3g}"
+    lim = 2e-4 if dtype == "float32" else 0.12
+    assert err.max() < lim, f"relative logit error {err.max():.3g} at row {int(err.argmax())}"
+
+
+def replay(eng, rid, toks, cuts):
+    """Feed ``toks`` of request ``rid`` in portions of the sizes ``cuts`` (cycled); all logits."""
+    out, i, k = [], 0, 0
+    while i < len(toks):
+        n = min(cuts[k % len(cuts)], len(toks) - i)
+        out.append(eng.replay_step([(rid, toks[i:i + n], list(range(n)))]))
+        i += n
+        k += 1
+    return np.concatenate(out)
+
+
+def tokens(n, vocab, seed):
+    return np.random.default_rng(seed).integers(0, vocab, n).tolist()
+
+
+def want_logits(cfg, params, toks, layers=None):
+    return oracle.forward(cfg, params, toks, layers).numpy()
+
+
+def decided_rows(cfg, params, toks, gap=0.03):
+    """Rows whose routing is no close call in any layer: 16-bit rounding of a router's input can
+    choose another expert where two scores nearly tie, which is no fault of the engine."""
+    margins = []
+    oracle.forward(cfg, params, toks, None, margins)
+    keep = np.ones(len(toks), dtype=bool)
+    for m in margins:
+        keep &= m.numpy() > gap
+    assert keep.mean() > 0.5
+    return keep
+
+
+# ---- whole prompts, decoding, portions ----------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+def test_whole_prompt_matches_oracle(model_dir, device):
+    path, cfg, params = model_dir()
+    toks = tokens(75, cfg["vocab"], 1)
+    layers = []
+    want = want_logits(cfg, params, toks, layers)
+    eng = engine(path, device)
+    close(eng.replay_step([("a", toks, list(range(len(toks))))]), want)
+    eng.finish_request("a")
+    # sum of the streams after every layer, first tokens of the sequence included
+    from agentic_traffic_testing_amd.engine.scheduler import Batch
+    from agentic_traffic_testing_amd.engine.sequence import Sequence
+
+    seq = Sequence("b", toks, SamplingParams())
+    assert eng.scheduler.admit(seq, len(toks))
+    lo = []
+    eng.runner.execute_logits(Batch([seq], [0], [len(toks)], 0), [0], layer_out=lo)
+    assert len(lo) == len(layers)
+    for i, x in enumerate(lo):
+        assert torch.allclose(x.cpu().double(), layers[i], atol=3e-3, rtol=3e-4), i
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("order", ["a-", "g-", "ad", "ge", "ae"])
+def test_each_mechanism_alone(model_dir, device, order):
+    """One-layer models: each mixer without a feed-forward, then with each kind of it."""
+    path, cfg, params = model_dir("only_" + order, order=order)
+    toks = tokens(45, cfg["vocab"], 7)
+    close(replay(engine(path, device), "a", toks, [28, 1, 1, 2, 6]), want_logits(cfg, params, toks))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_then_token_by_token(model_dir, device, dtype):
+    """The window (21 keys) passes over the border between the prompt and the decoded tokens."""
+    path, cfg, params = model_dir()
+    toks = tokens(90, cfg["vocab"], 2)
+    got = replay(engine(path, device, dtype), "a", toks, [37] + [1] * 60)
+    keep = decided_rows(cfg, params, toks) if dtype != "float32" else slice(None)
+    close(got[keep], want_logits(cfg, params, toks)[keep], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[2], [3, 2, 17, 1, 2, 5], [16, 15, 1, 33], [1], [21, 22, 20]])
+def test_portions_of_any_size(model_dir, device, cuts):
+    path, cfg, params = model_dir()
+    toks = tokens(70, cfg["vocab"], 3)
+    close(replay(engine(path, device), "a", toks, cuts), want_logits(cfg, params, toks))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding(model_dir, device):
+    """Hundreds of single-token steps: the window leaves whole pages and decode partitions
+    behind, the recurrent state and the shift rows are carried through every step."""
+    path, cfg, params = model_dir("long", order="adge", streams=2,
+                                  att=dict(ATT, mask={"size": 150}))
+    toks = tokens(330, cfg["vocab"], 4)
+    close(replay(engine(path, device), "a", toks, [3] + [1] * 400), want_logits(cfg, params, toks))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_other_sizes(model_dir, device):
+    """Values a model may happen to make equal or 1: one stream; one key / value head and as many
+    as query heads; rotation of the whole head, none, and without scaling; no window and a
+    window of one key; every expert chosen and a single one; widths that are not multiples of 8."""
+    variants = {
+        "one": dict(order="a-gea-", streams=1, width=40,
+                    att={"heads": 3, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 0.3,
+                         "rot": {"dims": 16, "base": 100.0}},
+                    moe={"kind": "moe", "expert": {"ff": 16, "limit": 0.6},
+                         "router": {"experts": 3, "top": 3}}),
+        "mha": dict(order="adgdae", streams=4, width=36, ff=20,
+                    att={"heads": 3, "kv_heads": 3, "dim": 10, "vdim": 10, "scale": 0.5,
+                         "mask": {"size": 1}},
+                    gru={"width": 7},
+                    moe={"kind": "moe", "expert": {"ff": 9, "limit": 30.0},
+                         "router": {"experts": 7, "top": 1}}),
+        "wide": dict(order="aegd", streams=2, width=64, ff=72,
+                     att={"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.11,
+                          "mask": {"size": 64},
+                          "rot": {"dims": 64, "base": 20000.0,
+                                  "scaling": {"factor": 2.0, "low": 2.0, "high": 8.0,
+                                              "original": 64}}},
+                     gru={"width": 130},
+                     moe={"kind": "moe", "expert": {"ff": 32, "limit": 2.5},
+                          "router": {"experts": 4, "top": 2}}),
+    }
+    for key, kw in variants.items():
+        path, cfg, params = model_dir(key, **kw)
+        toks = tokens(83, cfg["vocab"], 5)
+        close(replay(engine(path, device), "a", toks, [65, 1, 1, 2, 7]),
+              want_logits(cfg, params, toks))
+
+
+@pytest.mark.gpu
+def test_matrix_core_paths_in_bfloat16(model_dir):
+    """bf16 on the GPU with widths the matrix-core attention and expert kernels take."""
+    path, cfg, params = model_dir("wide", order="aegd", streams=2, width=64, ff=72)  # made above
+    toks = tokens(200, cfg["vocab"], 6)
+    got = replay(engine(path, "cuda", "bfloat16"), "a", toks, [130, 3] + [1] * 80)
+    keep = decided_rows(cfg, params, toks)
+    close(got[keep], want_logits(cfg, params, toks)[keep], "bfloat16")
+
+
+# ---- batches, pages and slots ---------------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+def test_mixed_batches_equal_each_alone(model_dir, device):
+    path, cfg, params = model_dir()
+    V = cfg["vocab"]
+    reqs = {"a": tokens(61, V, 10), "b": tokens(1, V, 11), "c": tokens(34, V, 12),
+            "d": tokens(50, V, 13), "e": tokens(23, V, 14)}
+    want = {k: want_logits(cfg, params, t) for k, t in reqs.items()}
+    # four live requests at most; 'e' arrives after 'b' and 'c' ended and reuses a slot and
+    # pages (the pool holds 10 pages of 16 tokens: everything is used again)
+    plan = [[("a", 17), ("b", 1)], [("a", 2), ("c", 30), ("d", 1)], [("a", 1), ("c", 1), ("d", 16)],
+            [("a", 1), ("c", 3), ("d", 2), ("e", 5)], [("a", 40), ("d", 31), ("e", 1)],
+            [("e", 17)]]
+    ends = {0: ["b"], 3: ["c"], 4: ["a", "d"], 5: ["e"]}
+    eng = engine(path, device, pool_tokens=160, max_seqs=4)
+    at = {k: 0 for k in reqs}
+    got = {k: [] for k in reqs}
+    for i, step in enumerate(plan):
+        portions = []
+        for rid, n in step:
+            portions.append((rid, reqs[rid][at[rid]:at[rid] + n], list(range(n))))
+            at[rid] += n
+        out = eng.replay_step(portions)
+        r = 0
+        for rid, n in step:
+            got[rid].append(out[r:r + n])
+            r += n
+        for rid in ends.get(i, []):
+            eng.finish_request(rid)
+    assert eng.runner.bm.num_free_state_slots() == 4
+    assert eng.runner.bm.num_free_blocks() == 10
+    for k in reqs:
+        assert at[k] == len(reqs[k])
+        close(np.concatenate(got[k]), want[k])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_freed_slot_and_pages_start_clean(model_dir, device):
+    """One slot, pages for one request: the next request inherits the slot and the pages with
+    the recurrent state, the shift rows and the keys of the one before still in them."""
+    path, cfg, params = model_dir()
+    eng = engine(path, device, pool_tokens=64, max_seqs=1)
+    for seed, n, cuts in ((20, 60, [60]), (21, 7, [1, 1, 5]), (22, 33, [2, 31]), (23, 1, [1])):
+        toks = tokens(n, cfg["vocab"], seed)
+        got = replay(eng, f"r{seed}", toks, cuts)
+        eng.finish_request(f"r{seed}")
+        close(got, want_logits(cfg, params, toks))
+
+
+def test_cache_layout(model_dir):
+    path, cfg, _ = model_dir()
+    eng = engine(path, "cpu")
+    layers = eng.runner.cache.layers
+    assert layers[0].k.shape[1:] == (ATT["kv_heads"], 16, ATT["dim"])
+    assert layers[0].v.shape[1:] == (ATT["kv_heads"], ATT["dim"], 16)
+    assert layers[1].state.shape[1:] == (1, 1, GRU["width"]) and layers[1].k is None
+    for lc in layers:
+        assert lc.shift.shape == (4, cfg["width"]) and lc.shift.dtype == torch.float32
+
+
+# ---- generation through the engine's own entry point ----------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation(model_dir, device):
+    path, cfg, params = model_dir()
+    prompts = [tokens(19, cfg["vocab"], 30), tokens(3, cfg["vocab"], 31), tokens(33, cfg["vocab"], 32)]
+    eng = engine(path, device)
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    outs = eng.generate(prompts, sp)
+    for p, o in zip(prompts, outs):
+        ids = list(p)
+        for tok in o.token_ids:
+            lg = oracle.forward(cfg, params, ids)[-1]
+            top2 = torch.topk(lg, 2).values
+            if float(top2[0] - top2[1]) > 1e-3:   # skip numerically tied steps
+                assert tok == int(lg.argmax())
+            ids.append(tok)
+        assert len(o.token_ids) == 12
+    assert eng.runner.bm.num_free_state_slots() == eng.runner.bm.num_state_slots()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_graph_replayed_decode_equals_eager(model_dir, dtype):
+    """Decode steps replayed from captured hipGraphs (several buckets, many replays with eager
+    prefill steps between them) give the tokens of the eager engine: the expert plan is made on
+    the device, so the routed layers are part of the graph."""
+    path, cfg, params = model_dir()
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (21, 2, 40)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        c = EngineConfig(model=path, device="cuda", dtype=dtype, max_model_len=512,
+                         max_num_seqs=4, max_num_batched_tokens=512, num_kv_blocks=64,
+                         use_graphs=graphs, graph_batch_sizes=(1, 2, 4), startup_warmup=False,
+                         gemm_tuning="")
+        eng = LLMEngine(c)
+        first = eng.generate(prompts, sp)
+        again = eng.generate(prompts[:2], sp)          # slots and pages reused, graphs replayed
+        outs[graphs] = [o.token_ids for o in first + again]
+        assert (eng.runner.graph_steps > 0) == graphs
+    if dtype == "float32":
+        assert outs[True] == outs[False]
+    assert outs[True][:2] == outs[True][3:]            # same prompts, same tokens the second time
+
+
+def test_registry_and_config_reader(model_dir):
+    path, cfg, _ = model_dir()
+    eng = engine(path, "cpu")
+    assert type(eng.runner.model).__name__ == "SemezenModel"
+    mc = eng.model_cfg
+    assert mc.hidden_size == cfg["width"] and mc.vocab_size == cfg["vocab"]
+    assert mc.streams == 3 and mc.rms_norm_eps == 3e-6
+    assert [L.kind for L in mc.layers] == ["attention", "mingru", "attention"]
+    a = mc.layers[0].mixer
+    assert (a.heads, a.kv_heads, a.dim, a.window, a.rot_dims) == (4, 2, 32, 21, 12)
+    assert a.rot_scaling == (6.0, 1.0, 3.0, 40.0) and a.scale == 0.21
+    assert mc.layers[0].ff == 40 and mc.layers[0].moe is None
+    m = mc.layers[1].moe
+    assert (m.experts, m.top, m.ff, m.limit) == (5, 2, 24, 1.25) and mc.layers[1].ff == 0
+    bad = json.loads(json.dumps(cfg))
+    bad["layers"][0]["mixer"]["vdim"] = 16          # the values are the keys
+    with pytest.raises(ValueError):
+        SemezenConfig.from_dict(bad)
+    bad = json.loads(json.dumps(cfg))
+    bad["layers"][1]["mlp"]["router"]["top"] = 6
+    with pytest.raises(ValueError):
+        SemezenConfig.from_dict(bad)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_preempted_sequence_recomputes_from_the_zero_state(model_dir, device):
+    path, cfg, _ = model_dir()
+    prompts = [tokens(20, cfg["vocab"], 70), tokens(18, cfg["vocab"], 71)]
+    sp = SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True)
+    want = [o.token_ids for o in engine(path, device, pool_tokens=512).generate(prompts, sp)]
+    small = engine(path, device, pool_tokens=80, max_seqs=2)
+    got = [o.token_ids for o in small.generate(prompts, sp)]
+    assert small.scheduler.num_preemptions > 0
+    assert got == want
+    assert small.runner.bm.num_free_state_slots() == 2
+
+
+def test_trace_replay_command_line(model_dir, tmp_path):
+    import os
+    import subprocess
+    import sys
+
+    path, cfg, params = model_dir()
+    V = cfg["vocab"]
+    a, b = tokens(30, V, 50), tokens(9, V, 51)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": [7]},
+                                {"id": "a", "tokens": a[11:12], "want": [0]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[8:], "want": []}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[12:], "want": [17]}], "end": ["a"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path,
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "128",
+                        "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                       capture_output=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == \
+        [f"done {i}" for i in range(4)]
+    wa, wb = want_logits(cfg, params, a), want_logits(cfg, params, b)
+    got = {i: np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V) for i in (0, 1, 3)}
+    assert not (out / "2.f32").exists()
+    close(got[0], wa[[0, 10]])
+    close(got[1], np.stack([wb[7], wa[11]]))
+    close(got[3], wa[[29]])
+
+
+# ---- mechanisms alone, made so that a fault shows ---------------------------------------------
+def i32(a, device):
+    return torch.tensor(np.asarray(a), dtype=torch.int32, device=device)
+
+
+def meta(lens, starts, slots, device):
+    pos = [s + j for n, s in zip(lens, starts) for j in range(n)]
+    qs = np.concatenate([[0], np.cumsum(lens)])
+    return i32(pos, device), i32(qs, device), i32(slots, device)
+
+
+def paged(k, v, bs, device, seed=0):
+    """Scatter a sequence's keys [T, G, d] and values [T, G, dv] into shuffled pages."""
+    T, G, d = k.shape
+    nblk = -(-T // bs)
+    perm = np.random.default_rng(seed).permutation(nblk + 2)
+    kc = torch.full((nblk + 2, G, bs, d), 7.0)
+    vc = torch.full((nblk + 2, G, v.shape[2], bs), -9.0)
+    for t in range(T):
+        kc[perm[t // bs], :, t % bs] = k[t]
+        vc[perm[t // bs], :, :, t % bs] = v[t]
+    return kc.to(device), vc.to(device), i32(perm[:nblk][None], device)
+
+
+def attend(q, kc, vc, bt, T, n, window, scale, device, decode=False):
+    """The last ``n`` rows of a ``T``-token sequence attend through the op layer."""
+    tiles = list(range(0, n, mx.ATTN_TILE_TOKENS))
+    if decode:
+        assert n == 1
+        return mx.sink_attention(q, kc, vc, bt, i32([T], device), i32([0, 1], device),
+                                 i32([], device), i32([], device), scale, False, 1, T,
+                                 window=window)
+    return mx.sink_attention(q, kc, vc, bt, i32([T], device), i32([0, n], device),
+                             i32([0] * len(tiles), device), i32(tiles, device), scale, False,
+                             window=window)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,window", [(700, 300), (300, 129), (140, 17), (97, 64), (40, 1000)])
+def test_window_finds_one_key_at_its_edge(device, dtype, T, window):
+    """Among hundreds of random keys ONE has a large score with every query.  Placed on the last
+    key inside a row's window it takes all the weight; one step further out it must not be seen
+    at all.  Checked for the last row of a prompt portion and for a single decode row, with the
+    edge inside a page, at page borders and in another decode partition than the query."""
+    if device == "cpu" and dtype == torch.bfloat16:
+        pytest.skip("the CPU tier computes in fp32 either way")
+    H, G, d = 4, 2, 32
+    g = torch.Generator().manual_seed(T)
+    q = torch.randn(T, H, d, generator=g) * 0.3
+    k = torch.randn(T, G, d, generator=g) * 0.3
+    v = torch.randn(T, G, d, generator=g)
+    mark = torch.zeros(d)
+    mark[5] = 12.0
+    q[:, :, 5] = 12.0
+    scale = 0.5
+    inside = T - min(window, T)            # first key the last row still sees
+    for place in {inside, inside - 1, T - 1, 0} - {-1}:
+        kk = k.clone()
+        kk[place] = mark
+        ref = oracle.window_softmax_attention(q.double(), kk.double(), v.double(), scale, window)
+        kc, vc, bt = paged(kk.to(dtype).float(), v.to(dtype).float(), 16, device, seed=place)
+        kc, vc = kc.to(dtype), vc.to(dtype)
+        tol = 2e-4 if dtype == torch.float32 else 4e-2
+        for n in (1, min(T, 70)):
+            for decode in ((False, True) if n == 1 else (False,)):
+                got = attend(q[T - n:].to(dtype).to(device), kc, vc, bt, T, n, window, scale,
+                             device, decode)
+                assert torch.allclose(got.cpu().double(), ref[T - n:], atol=tol, rtol=tol), \
+                    (place, n, decode)
+        seen = inside <= place
+        w_last = torch.allclose(ref[T - 1, 0], v[place, 0].double(), atol=1e-3)
+        assert w_last == seen
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_rotation_scaled_partial_far_positions(device):
+    """Rotate-half pairs on 6 of 16 channels at positions up to 5000, scaled frequencies, the
+    norm after the rotation and without a weight; values are the unrotated, unnormed keys."""
+    H, G, d, T = 3, 1, 16, 6
+    rot = {"dims": 6, "base": 300.0, "scaling": {"factor": 5.0, "low": 1.0, "high": 2.0,
+                                                  "original": 30}}
+    g = torch.Generator().manual_seed(3)
+    qx, kx = torch.randn(T, H * d, generator=g), torch.randn(T, G * d, generator=g)
+    pos = torch.tensor([0, 1, 17, 300, 4999, 5000])
+    fr = oracle.rotary_frequencies(rot["dims"], rot["base"], rot["scaling"])
+    want_q = oracle.rms(oracle.rotate(qx.double().view(T, H, d), pos, fr), 1e-6)
+    want_k = oracle.rms(oracle.rotate(kx.double().view(T, G, d), pos, fr), 1e-6)
+    inv = mx.scaled_inv_freq(6, 300.0, (5.0, 1.0, 2.0, 30.0), device)
+    assert torch.allclose(inv.cpu().double(), fr, rtol=1e-6)
+    assert fr[0] == 1.0 and abs(fr[2] - 300.0 ** (-4 / 6) / 5.0) < 1e-12   # kept / slowed down
+    tab = mx.rotary_table(i32(pos, device), inv)
+    kc = torch.zeros(2, G, 16, d, device=device)
+    vc = torch.zeros(2, G, d, 16, device=device)
+    slots = i32([3, 4, 20, 21, 31, 0], device)
+    q = mx.qk_norm_rope_cache(qx.to(device), kx.to(device), kx.to(device), None, None, 1e-6,
+                              i32(pos, device), slots, tab, kc, vc, H, G, d, d,
+                              rotate_half_pairs=True, norm_last=True)
+    assert torch.allclose(q.cpu().double(), want_q, atol=2e-3)      # fp32 angles at 5000
+    for t, s in enumerate(slots.tolist()):
+        assert torch.allclose(kc[s // 16, :, s % 16].cpu().double(), want_k[t], atol=2e-3)
+        assert torch.equal(vc[s // 16, :, :, s % 16].cpu(), kx[t].view(G, d))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_token_shift_across_portions_and_slots(device):
+    W = 24
+    g = torch.Generator().manual_seed(5)
+    n = torch.randn(11, W, generator=g)
+    mu = torch.rand(W, generator=g)
+    want = oracle.token_shift(n.double(), mu)
+    state = torch.full((3, W), 1e6)                 # poisoned: position 0 must not read it
+    other = torch.randn(4, W, generator=g)
+    got = []
+    # sequence in slot 2 in portions of 1, 4, 1, 5 rows, next to another sequence in slot 0
+    at = 0
+    for step, cnt in enumerate((1, 4, 1, 5)):
+        rows = torch.cat([other[step:step + 1], n[at:at + cnt]]).to(device)
+        pos, qs, sl = meta([1, cnt], [step, at], [0, 2], device)
+        st = state.to(device) if step == 0 else st
+        out = mx.token_shift(rows, mu.to(device), st, pos, qs, sl, torch.float32)
+        got.append(out[1:].cpu())
+        at += cnt
+    assert torch.allclose(torch.cat(got).double(), want, atol=1e-5)
+    assert torch.allclose(st[2].cpu(), n[-1]) and torch.allclose(st[0].cpu(), other[3])
+    assert float(st[1].min()) == 1e6                # a slot nobody owns is not touched
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_mingru_state_across_portions(device):
+    """Portions shorter and longer than a scan segment, a poisoned slot, a gate that is shut
+    (the state must survive hundreds of tokens) and one that is wide open."""
+    C, T = 40, 420
+    g = torch.Generator().manual_seed(6)
+    z, x, gt = (torch.randn(T, C, generator=g) * 2 for _ in range(3))
+    z[:, 0] = -40.0          # shut after the first token writes nothing: state stays 0
+    z[0, 1], z[1:, 1] = 40.0, -40.0     # written once, then kept
+    z[:, 2] = 40.0           # follows the candidate
+    gate = torch.sigmoid(z.double())
+    cand = torch.where(x.double() >= 0, x.double() + 0.5, torch.sigmoid(x.double()))
+    S = torch.zeros(C, dtype=torch.float64)
+    want = []
+    for t in range(T):
+        S = (1 - gate[t]) * S + gate[t] * cand[t]
+        want.append(S * (gt[t].double() * torch.sigmoid(gt[t].double())))
+    want = torch.stack(want)
+    state = torch.full((2, 1, 1, C), -1e5).to(device)
+    got, at = [], 0
+    for cnt in (1, 2, 300, 1, 1, 17, 98):
+        pos, qs, sl = meta([cnt], [at], [1], device)
+        got.append(mx.mingru_scan(z[at:at + cnt].to(device), x[at:at + cnt].to(device),
+                                  gt[at:at + cnt].to(device), state, pos, qs, sl,
+                                  torch.float32).cpu())
+        at += cnt
+    got = torch.cat(got).double()
+    assert torch.allclose(got, want, atol=2e-5, rtol=2e-5)
+    assert torch.allclose(state[1, 0, 0].cpu().double(), S, atol=2e-5)
+    assert abs(float(state[1, 0, 0, 1]) - float(cand[0, 1])) < 1e-6
+    assert float(state[0].max()) == -1e5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_expert_weight_scales_the_input(device):
+    """With the clamps active, scaling the expert's input differs from scaling its output; the
+    chosen experts are the ones with the largest sigmoid scores and their weights are not
+    renormalised."""
+    T, W, E, ff, top, limit = 70, 24, 6, 16, 2, 0.8
+    g = torch.Generator().manual_seed(8)
+    h = torch.randn(T, W, generator=g)
+    st = {"router": torch.randn(E, W, generator=g)}
+    for e in range(E):
+        st[f"e{e}.gate"] = torch.randn(ff, W, generator=g) * 0.6
+        st[f"e{e}.up"] = torch.randn(ff, W, generator=g) * 0.6
+        st[f"e{e}.down"] = torch.randn(W, ff, generator=g) * 0.3
+    mlp = {"router": {"experts": E, "top": top}, "expert": {"ff": ff, "limit": limit}}
+    want = oracle.moe_ff(h.double(), mlp, st, "")
+    logits = (h @ st["router"].T).to(device)
+    idx, wts = mx.moe_route(logits, top)
+    sc = torch.sigmoid(logits.cpu().double())
+    assert torch.equal(idx.cpu().long().sort(1).values, sc.topk(top, 1).indices.sort(1).values)
+    assert torch.allclose(wts.cpu().double().sum(1), sc.topk(top, 1).values.sum(1), atol=1e-6)
+    w_gu = torch.stack([torch.cat([st[f"e{e}.gate"], st[f"e{e}.up"]]) for e in range(E)])
+    w_down = torch.stack([st[f"e{e}.down"] for e in range(E)])
+    got = mx.moe_experts(h.to(device), idx, wts, w_gu.to(device), w_down.to(device), limit, 1.702)
+    assert torch.allclose(got.cpu().double(), want, atol=2e-4, rtol=2e-4)
+    # the other reading (weight on the output) is far from it
+    other = torch.zeros_like(want)
+    for t in range(T):
+        for e in sc[t].topk(top).indices.tolist():
+            other[t] += sc[t, e] * oracle.expert(h[t].double(), st, f"e{e}.", limit)
+    assert float((other - want).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_streams_mix_from_to(device):
+    """x_t = sum_s mix[s, t] x_s + out[t] y with a strongly asymmetric mix."""
+    T, s, W = 5, 3, 20
+    g = torch.Generator().manual_seed(9)
+    xs = torch.randn(T, s, W, generator=g)
+    y = torch.randn(T, W, generator=g)
+    mix = torch.tensor([[1.0, 2.0, 0.0], [0.0, 1.0, -3.0], [0.5, 0.0, 1.0]])
+    w_out, w_in = torch.tensor([1.0, -2.0, 0.25]), torch.tensor([0.3, 0.0, -1.0])
+    w = torch.rand(W, generator=g) + 0.5
+    want_x = torch.stack([sum(mix[a, t] * xs[:, a] for a in range(s)) + w_out[t] * y
+                          for t in range(s)], 1)
+    u = sum(w_in[t] * want_x[:, t] for t in range(s)).double()
+    want_n = oracle.rms_norm(u, w, 1e-6)
+    xd = xs.clone().to(device)
+    n = mx.hyper_update_norm(xd, y.to(device), mix.to(device), w_out.to(device), w_in.to(device),
+                             w.to(device), 1e-6, torch.float32)
+    assert torch.allclose(xd.cpu(), want_x, atol=1e-5)
+    assert torch.allclose(n.cpu().double(), want_n, atol=1e-5)
