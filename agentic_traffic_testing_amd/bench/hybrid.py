@@ -1,12 +1,12 @@
-"""Prefill and decode throughput of the hybrid decoders (Ledazen, Soselix) next to the models of
-the same layer geometry - Llama, and for Soselix also Ledazen, the closest family (softmax +
-recurrent mixers on the same cache and kernels) - through the serving engine (scheduler, paged
-cache / state slots, kernels).
+"""Prefill and decode throughput of the hybrid decoders (Ledazen, Soselix, Semezen) next to the
+models of the same layer geometry - Llama, and for Soselix and Semezen also the closest earlier
+hybrid family (softmax + recurrent mixers on the same cache and kernels) - through the serving
+engine (scheduler, paged cache / state slots, kernels).
 
 Random-init weights, synthetic token ids.  Per model and shape:
   prefill  - B prompts of P tokens admitted together, one generated token each: prompt tok/s
   decode   - the same B sequences generating N more tokens: generated tok/s
-``python bench.py --hybrid [ledazen|soselix]`` prints one JSON line per measurement.
+``python bench.py --hybrid [ledazen|soselix|semezen]`` prints one JSON line per measurement.
 """
 from __future__ import annotations
 
@@ -20,7 +20,10 @@ PAIRS = (("ledazen-small", "small"), ("ledazen-3b-slice", "llama-3b-slice"),
 SOSELIX = (("soselix-small", "ledazen-small", "small"),
            ("soselix-3b-slice", "ledazen-3b-slice", "llama-3b-slice"),
            ("soselix-8b-slice", "ledazen-8b-slice", "llama-8b-slice"))
-FAMILIES = {"ledazen": PAIRS, "soselix": SOSELIX}
+SEMEZEN = (("semezen-small", "soselix-small", "small"),
+           ("semezen-3b-slice", "soselix-3b-slice", "llama-3b-slice"),
+           ("semezen-8b-slice", "soselix-8b-slice", "llama-8b-slice"))
+FAMILIES = {"ledazen": PAIRS, "soselix": SOSELIX, "semezen": SEMEZEN}
 
 
 def _engine(model: str, device: str, dtype: str, max_len: int, seqs: int, budget: int):
