@@ -245,6 +245,13 @@ def test_matrix_core_paths_in_bfloat16(model_dir):
     got = replay(engine(path, "cuda", "bfloat16"), "a", toks, [130, 3] + [1] * 80)
     keep = decided_rows(cfg, params, toks)
     close(got[keep], want_logits(cfg, params, toks)[keep], "bfloat16")
+    # a 150-key window over a 200-token portion, then decode rows whose window crosses the
+    # 128- and 256-key partition borders
+    path, cfg, params = model_dir("long", order="adge", streams=2, att=dict(ATT, mask={"size": 150}))
+    toks = tokens(330, cfg["vocab"], 8)
+    got = replay(engine(path, "cuda", "bfloat16"), "b", toks, [200] + [1] * 130)
+    keep = decided_rows(cfg, params, toks)
+    close(got[keep], want_logits(cfg, params, toks)[keep], "bfloat16")
 
 
 # ---- batches, pages and slots ---------------------------------------------------------------
