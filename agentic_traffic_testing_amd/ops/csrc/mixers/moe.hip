@@ -21,9 +21,10 @@
 //   Matrix-core kernel (bf16, K % 8 == 0): mfma_f32_32x32x16_bf16 with the weights as the A operand
 //   (features = accumulator rows, so a lane holds 4 consecutive features of one row of the
 //   output), 4 waves = 2 x 2, K in steps of 64 through LDS with the next step's loads in flight;
-//   tiles of 64 x 64 for steps of few rows (they stream the weights once) and 128 x 128 (four
-//   32 x 32 blocks per wave) for prefill-sized steps, where the operand traffic per product
-//   decides.  Rows kernel (any dtype and sizes): fp32 FMA, 4 x 4 outputs per thread from fp32
+//   tiles of 64 features x 64 rows for steps of few rows (they stream the weights once); for
+//   prefill-sized steps, where the operand traffic per product decides, 128 rows x 128 features
+//   (four 32 x 32 blocks per wave) in the plain form and 128 rows x 64 features of gate and of
+//   up in the GLU form (the same four blocks per wave and LDS per workgroup).  Rows kernel (any dtype and sizes): fp32 FMA, 4 x 4 outputs per thread from fp32
 //   LDS tiles of 64 rows x 64 features.
 // * clamped_glu (rows of [gate | up] products from library GEMMs), pair_sum (a row's choices and
 //   split partials added in fp32).
@@ -473,11 +474,13 @@ extern "C" int mixk_moe_experts(void* y, void* act, int* plan, const void* h, co
   const int k_chunk = split > 1 ? ((ff + split - 1) / split + kMoeBK - 1) / kMoeBK * kMoeBK : ff;
   MoeArgs a2{plan, wts, max_tiles, top, W, ff, static_cast<int64_t>(ff),
              static_cast<int64_t>(W) * ff, limit, alpha, split, k_chunk};
-  const int ft = tile_rows == 128 ? 128 : kMoeFeat;
-  const dim3 g1(max_tiles, (ff + ft - 1) / ft), g2(max_tiles, (W + ft - 1) / ft);
+  // feature blocks: 64 for the gate | up form (two weight tiles per block), 128 for the down form
+  // of the large tiles
+  const int ft2 = tile_rows == 128 && mfma ? 128 : kMoeFeat;
+  const dim3 g1(max_tiles, (ff + kMoeFeat - 1) / kMoeFeat), g2(max_tiles, (W + ft2 - 1) / ft2);
 #define MIXK_MOE_MFMA(MF, MR, YT, GZ)                                                             \
   do {                                                                                            \
-    hipLaunchKernelGGL((moe_gemm_mfma_kernel<true, MF, MR, __bf16>), g1, dim3(256), 0, st,        \
+    hipLaunchKernelGGL((moe_gemm_mfma_kernel<true, 1, MR, __bf16>), g1, dim3(256), 0, st,         \
                        static_cast<__bf16*>(act), static_cast<const __bf16*>(h),                  \
                        static_cast<const __bf16*>(w_gate), static_cast<const __bf16*>(w_up), a1); \
     hipLaunchKernelGGL((moe_gemm_mfma_kernel<false, MF, MR, YT>), dim3(g2.x, g2.y, GZ), dim3(256), \
