@@ -596,6 +596,180 @@ HYBRID_PRESETS.update({
 ARCHITECTURES["Semezen"] = SemezenConfig.from_dict
 
 
+# ---------------------------------------------------------------------------------------
+# Lovapel: decoder with a layer norm before AND after every sub-layer, sliding-window attention
+# with a learned sink per head and q / k norms over the whole projection, dense GELU-GLU layers or
+# grouped-choice routed experts (with identity experts and a shared expert), a span of layers
+# that runs several times with the same weights, tied and soft-capped output logits.
+
+@dataclass(frozen=True)
+class SinkWindowAttentionConfig:
+    """Grouped-query softmax attention: q and k RMS-normed over their WHOLE projection (all heads
+    at once, one weight per row of the projection) before the rotation, rotate-half positions on
+    the first ``rot_dims`` channels of every head, a sliding window of ``window`` keys (0: all
+    earlier keys) and one learned sink score per query head in the softmax denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+
+
+@dataclass(frozen=True)
+class GroupedMoeConfig:
+    """``experts`` SiLU-GLU feed-forward layers of width ``ff`` plus ``identity`` experts without
+    weights that return their input.  The router's softmax scores (plus a stored correction,
+    used for the choice only) pick ``top`` experts inside the ``keep`` best of ``groups`` equal
+    runs of neighbours; the chosen scores, normalised to sum 1, weight the outputs.  A shared
+    expert of width ``shared_ff`` (0: none) runs for every token."""
+    experts: int
+    top: int
+    ff: int
+    identity: int = 0
+    groups: int = 1
+    keep: int = 1
+    shared_ff: int = 0
+
+    @property
+    def routes(self) -> int:
+        return self.experts + self.identity
+
+
+@dataclass(frozen=True)
+class LovapelLayerConfig:
+    kind: str                 # "attention"
+    mixer: object = None
+    ff: int = 0               # dense GELU-GLU width (0: none, or see ``moe``)
+    moe: GroupedMoeConfig | None = None
+
+
+@dataclass(frozen=True)
+class LovapelConfig:
+    name: str = "lovapel"
+    vocab_size: int = 1024
+    hidden_size: int = 256
+    layers: tuple = ()
+    norm_eps: float = 1e-5
+    loop_start: int = 0       # layers [loop_start, loop_stop) run loop_times times in a row
+    loop_stop: int = 0
+    loop_times: int = 1
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0   # 0: none
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    max_position_embeddings: int = 1 << 20
+    family: str = "lovapel"
+
+    @property
+    def runs(self) -> tuple:
+        """Layer index of every layer run, in order; a run has a cache of its own."""
+        a, b = self.loop_start, self.loop_stop
+        n = len(self.layers)
+        return tuple(range(a)) + tuple(range(a, b)) * self.loop_times + tuple(range(b, n))
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.runs)
+
+    @property
+    def rms_norm_eps(self) -> float:
+        return self.norm_eps
+
+    def __post_init__(self):
+        n = len(self.layers)
+        if not (0 <= self.loop_start <= self.loop_stop <= n) or self.loop_times < 1:
+            raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 1")
+
+    @staticmethod
+    def from_dict(c: dict, name: str = "lovapel") -> "LovapelConfig":
+        """Parse the checkpoint's config.json (keys: vocab, width, norm.eps, logit_scale,
+        logit_softcap, loop.{start, stop, times}, layers[].{type, mixer, mlp}; attention: heads,
+        kv_heads, dim, vdim, scale, mask.size, rot.{dims, base}; mlp: kind dense {ff} or moe
+        {expert.ff, router.{experts, identity, top, groups.{count, keep}}, shared.ff}).  An absent
+        loop, mask, rot, softcap, groups, identity or shared means none."""
+        layers = []
+        for i, L in enumerate(c["layers"]):
+            m, t = L["mixer"], L["type"]
+            if t != "attention":
+                raise ValueError(f"unknown layer type {t!r}")
+            rot = m.get("rot") or {}
+            mc = SinkWindowAttentionConfig(
+                heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                window=int((m.get("mask") or {}).get("size") or 0),
+                rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)))
+            if mc.heads % mc.kv_heads:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            if mc.rot_dims % 2 or mc.rot_dims > mc.dim:
+                raise ValueError(f"layer {i}: rot.dims must be even and <= dim")
+            mlp = L.get("mlp")
+            ff, moe = 0, None
+            if mlp:
+                kind = str(mlp.get("kind", "dense"))
+                if kind == "dense":
+                    ff = int(mlp["ff"])
+                elif kind == "moe":
+                    r = mlp["router"]
+                    g = r.get("groups") or {}
+                    groups = int(g.get("count", 1))
+                    moe = GroupedMoeConfig(
+                        experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                        identity=int(r.get("identity", 0)), groups=groups,
+                        keep=int(g.get("keep", groups)),
+                        shared_ff=int((mlp.get("shared") or {}).get("ff", 0)))
+                    if moe.groups < 1 or moe.routes % moe.groups:
+                        raise ValueError(f"layer {i}: the experts do not split into equal groups")
+                    if not 1 <= moe.keep <= moe.groups:
+                        raise ValueError(f"layer {i}: groups.keep must be in [1, groups.count]")
+                    if not 1 <= moe.top <= moe.keep * (moe.routes // moe.groups):
+                        raise ValueError(f"layer {i}: router.top exceeds the experts of the kept groups")
+                else:
+                    raise ValueError(f"unsupported feed-forward kind {kind!r}")
+            layers.append(LovapelLayerConfig(t, mc, ff, moe))
+        loop = c.get("loop") or {}
+        return LovapelConfig(
+            name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+            layers=tuple(layers), norm_eps=float(c["norm"]["eps"]),
+            loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+            loop_times=int(loop.get("times", 1)), logit_scale=float(c.get("logit_scale", 1.0)),
+            logit_softcap=float(c.get("logit_softcap") or 0.0))
+
+
+def lovapel_preset(name: str, vocab: int, width: int, ff: int, pattern: str, heads: int,
+                   kv_heads: int, dim: int, window: int, experts: int = 8, top: int = 2,
+                   expert_ff: int = 0, identity: int = 0, groups: int = 1, keep: int = 1,
+                   shared_ff: int = 0, loop: tuple = (0, 0, 1)) -> LovapelConfig:
+    """A Lovapel shape for benchmarks and tests: one letter per layer for its feed-forward
+    (``d`` dense, ``e`` experts, ``-`` none); every mixer is the sink-window attention."""
+    mc = SinkWindowAttentionConfig(heads, kv_heads, dim, dim, dim ** -0.5, window, dim // 2,
+                                   500000.0)
+    layers = tuple(LovapelLayerConfig(
+        "attention", mc, ff if f == "d" else 0,
+        GroupedMoeConfig(experts, top, expert_ff or max(8, ff // max(1, top)), identity, groups,
+                         keep, shared_ff) if f == "e" else None) for f in pattern)
+    return LovapelConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers,
+                         loop_start=loop[0], loop_stop=loop[1], loop_times=loop[2],
+                         logit_scale=0.5, logit_softcap=30.0)
+
+
+HYBRID_PRESETS.update({
+    "lovapel-tiny": lovapel_preset("lovapel-tiny", 512, 128, 192, "ded", 4, 2, 32, 24, 6, 2, 48,
+                                   2, 4, 2, 40, (1, 3, 2)),
+    # the "small" Llama preset's geometry (width 1024, 8 q / 2 kv heads of 128, FFN 2816, 4 layers)
+    "lovapel-small": lovapel_preset("lovapel-small", 32768, 1024, 2816, "dede", 8, 2, 128, 1024,
+                                    8, 2, 1408, 0, 2, 1, 704),
+    # Llama-3.2-3B / Llama-3.1-8B layer geometry, one dense layer and one with experts
+    "lovapel-3b-slice": lovapel_preset("lovapel-3b-slice", 16384, 3072, 8192, "de", 24, 8, 128,
+                                       1024, 8, 2, 4096, 0, 2, 1, 2048),
+    "lovapel-8b-slice": lovapel_preset("lovapel-8b-slice", 16384, 4096, 14336, "de", 32, 8, 128,
+                                       1024, 8, 2, 7168, 0, 2, 1, 3584),
+})
+ARCHITECTURES["Lovapel"] = LovapelConfig.from_dict
+
+
 def resolve_model(model: str) -> tuple[ModelConfig, str | None]:
     """Map a reference-style model id (``meta-llama/Llama-3.1-8B-Instruct``), a preset name
     or a local HF directory (config.json [+ *.safetensors]) to a ModelConfig.

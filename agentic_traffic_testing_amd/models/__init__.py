@@ -19,7 +19,11 @@ def model_class(family: str):
         from .semezen import SemezenModel
 
         return SemezenModel
+    if family == "lovapel":
+        from .lovapel import LovapelModel
+
+        return LovapelModel
     raise ValueError(f"no model registered for family {family!r}")
 
 
-FAMILIES = ("llama", "ledazen", "soselix", "semezen")
+FAMILIES = ("llama", "ledazen", "soselix", "semezen", "lovapel")

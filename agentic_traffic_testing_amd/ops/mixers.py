@@ -4,8 +4,11 @@ an optional sink (score 0 or one learned score per head); latent attention's fro
 short causal convolutions with carried tails; the gated delta rule and the gated linear
 recurrence (forget-gate and state-space forms) with per-sequence fp32 state; the fp32-residual
 norms, sums and activations around them; hyper-connection streams, token shift, the minGRU
-recurrence, element-wise gates, GELU, and routed clamped-GLU experts (grouped matrix products
-over rows sorted by expert).
+recurrence, element-wise gates, GELU, and routed clamped-GLU or SiLU-GLU experts (grouped matrix
+products over rows sorted by expert; sigmoid or softmax routing, optionally with a choice
+correction and group-limited choice; identity experts), the sandwich-norm layer boundary (layer
+norm or RMS norm of a branch added to the fp32 residual, then the next norm), q / k norms over
+a whole projection, and scaled, soft-capped logits.
 
 Same device-strict dispatch as ``ops``: GPU tensors run the HIP kernels of
 ``ops/csrc/mixers`` (library ``_atta_mixers.so``, operators ``torch.ops.atta_mix.*``; built on
@@ -69,7 +72,8 @@ def _native():
 ATTN_TILE_TOKENS = 64     # query tokens per prefill attention tile (the block manager tiles by it)
 DECODE_PART_TOKENS = 128  # keys per decode-attention partition
 ATTENTION_MFMA = os.environ.get("ATTA_MIX_ATTENTION_MFMA", "1") != "0"
-ACT_SILU, ACT_SIGMOID = 0, 1
+ACT_SILU, ACT_SIGMOID, ACT_GELU_TANH = 0, 1, 2
+_ACT_CODES = {"silu": ACT_SILU, "sigmoid": ACT_SIGMOID, "gelu_tanh": ACT_GELU_TANH}
 
 
 def inv_freq(rot_dims: int, base: float, device) -> torch.Tensor:
@@ -128,18 +132,26 @@ def rotary_table(positions, inv_freq_t):
 
 def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
                        k_cache, v_cache, heads, kv_heads, dim, vdim, rotate_half_pairs=False,
-                       norm_last=False):
+                       norm_last=False, whole_norm=False):
     """qx / kx / vx: row-strided [T, heads * dim] / [T, kv_heads * dim] / [T, kv_heads * vdim];
     cos_sin: ``rotary_table`` of the step's positions.  ``q_norm`` / ``k_norm`` None: the norm
     has no weight; ``rotate_half_pairs``: channel i pairs with i + n_freq instead of
-    (2i, 2i + 1); ``norm_last``: rotate first, then norm."""
+    (2i, 2i + 1); ``norm_last``: rotate first, then norm; ``whole_norm``: q (and k) are normed
+    over the whole projection, all heads at once, with weights [heads * dim] ([kv_heads * dim]) -
+    a one-wave-per-row kernel computes the two inverse root mean squares of every row first."""
     if not qx.is_cuda:
         return mref.qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
                                        cos_sin, k_cache, v_cache, heads, kv_heads, dim, vdim,
-                                       rotate_half_pairs, norm_last)
+                                       rotate_half_pairs, norm_last, whole_norm)
+    if whole_norm and norm_last:
+        raise ValueError("a norm over the whole projection precedes the rotation")
     q = torch.empty(qx.shape[0], heads, dim, dtype=qx.dtype, device=qx.device)
+    row_inv = None
+    if whole_norm:
+        row_inv = torch.empty(qx.shape[0], 2, dtype=torch.float32, device=qx.device)
+        _native().proj_inv_rms(row_inv, qx, kx, eps)
     _native().qk_norm_rope_cache(q, qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
-                                 cos_sin, k_cache, v_cache, rotate_half_pairs, norm_last)
+                                 cos_sin, k_cache, v_cache, rotate_half_pairs, norm_last, row_inv)
     return q
 
 
@@ -373,8 +385,9 @@ def token_shift(n, mu, shift_state, positions, seq_qstart, seq_slot, dtype=torch
 
 
 def gate_mul(a, gate, act="sigmoid"):
-    """a [T, N] times sigmoid / SiLU of the row-strided gate [T, N]."""
-    code = ACT_SIGMOID if act == "sigmoid" else ACT_SILU
+    """a [T, N] times sigmoid / SiLU / tanh-form GELU of the gate [T, N]; both may be row-strided
+    slices of a fused projection (a GLU is ``gate_mul(up, gate, act)``)."""
+    code = _ACT_CODES[act]
     if not a.is_cuda:
         return mref.gate_mul(a, gate, code)
     out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
@@ -430,60 +443,89 @@ def clamped_glu(gu, wts, limit, alpha=1.702):
     return out
 
 
-def _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha):
+def _moe_combine(y, idx, wts, h, addend, E, split):
+    """out[t] = sum_j wts[t, j] * (y[t, j] summed over its ``split`` partial rows, or h[t] for an
+    identity expert idx[t, j] >= E) (+ addend[t]), in fp32, stored in h's dtype."""
+    out = torch.empty_like(h)
+    _native().moe_combine(out, y, idx, wts, h, addend, E, split)
+    return out
+
+
+def _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha, silu_glu=False, addend=None):
     """Prefill-sized steps: rows sorted by expert, then per expert one library product with the
     stacked [gate; up] matrix, the activation kernel and one library product with the down
     matrix.  The per-expert row counts come to the host (one synchronisation per call), so this
     path is not taken while a graph is being recorded."""
     T, W = h.shape
     k = idx.shape[1]
+    E, ff = w_gu.shape[0], w_gu.shape[1] // 2
     flat = idx.flatten().long()
     order = torch.argsort(flat, stable=True)
-    counts = torch.bincount(flat, minlength=w_gu.shape[0]).tolist()
+    counts = torch.bincount(flat, minlength=E).tolist()
     xs = h.index_select(0, torch.div(order, k, rounding_mode="floor"))
     ws = wts.flatten().index_select(0, order)
     ys = torch.empty(T * k, W, dtype=h.dtype, device=h.device)
     off = 0
-    for e, c in enumerate(counts):
+    for e, c in enumerate(counts[:E]):     # indices >= E are identity experts: no product
         if c:
             gu = torch.nn.functional.linear(xs[off:off + c], w_gu[e])
-            torch.mm(clamped_glu(gu, ws[off:off + c], limit, alpha), w_down[e].t(),
-                     out=ys[off:off + c])
+            a = (gate_mul(gu[:, ff:], gu[:, :ff], "silu") if silu_glu else
+                 clamped_glu(gu, ws[off:off + c], limit, alpha))
+            torch.mm(a, w_down[e].t(), out=ys[off:off + c])
             off += c
     y = torch.empty_like(ys)
     y.index_copy_(0, order, ys)
+    if silu_glu:
+        return _moe_combine(y, idx, wts, h, addend, E, 1)
     return _pair_sum(y, T, k)
 
 
-def moe_route(logits, top):
-    """fp32 router logits [T, E] -> (expert index int32 [T, top], sigmoid score fp32 [T, top]) of
-    every row's ``top`` largest scores (ties: lowest index)."""
+def moe_route(logits, top, score="sigmoid", correction=None, groups=1, keep=1, renorm=False):
+    """fp32 router logits [T, E] -> (expert index int32 [T, top], score fp32 [T, top]) of every
+    row's ``top`` largest scores (ties: lowest index).  ``score``: "sigmoid", or "softmax" over
+    the row.  ``correction`` fp32 [E] is added to the scores for the choice only (the returned
+    weights are the plain scores).  ``groups`` > 1: the experts form that many equal runs of
+    neighbours, a group's score is its largest choice score, and only experts of the ``keep``
+    best groups can be chosen.  ``renorm``: the chosen scores are divided by their sum + 1e-20."""
+    E = logits.shape[1]
+    if groups < 1 or E % groups or not 1 <= keep <= groups or top > keep * (E // groups):
+        raise ValueError("moe_route: groups must split the experts evenly and hold `top` of them")
     if not logits.is_cuda:
-        return mref.moe_route(logits, top)
+        return mref.moe_route(logits, top, score == "softmax", correction, groups, keep, renorm)
     T = logits.shape[0]
     idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    _native().moe_route(idx, wts, logits)
+    _native().moe_route(idx, wts, logits, score == "softmax", correction, groups, keep, renorm)
     return idx, wts
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702):
-    """Routed clamped-GLU experts: out[t] = sum_j W_down[e] act(W_gate[e] (w h_t), W_up[e] (w h_t))
-    over the row's chosen (e, w) = (idx[t, j], wts[t, j]); act(g, u) = g' sigmoid(alpha g')
-    (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit).  w_gu [E, 2 ff, W] stacks every
-    expert's gate rows on its up rows; w_down [E, W, ff].  On the GPU: one planning kernel sorts
-    the (row, choice) pairs by expert into tiles of MOE_TILE_ROWS (or MOE_BIG_TILE_ROWS), then two
-    grouped matrix products (gate | up with the activation in the epilogue; down) run over the
-    tiles - no host synchronisation, so the step can be captured in a graph.  Steps whose expert
-    products reach MOE_LIBRARY_FLOPS run library products per expert instead (outside a capture)."""
+def moe_experts(h, idx, wts, w_gu, w_down, limit=0.0, alpha=1.702, glu="clamped", addend=None):
+    """Routed GLU experts over a row's chosen (e, w) = (idx[t, j], wts[t, j]); w_gu [E, 2 ff, W]
+    stacks every expert's gate rows on its up rows; w_down [E, W, ff].
+
+    ``glu`` "clamped": out[t] = sum_j W_down[e] act(W_gate[e] (w h_t), W_up[e] (w h_t)) - the
+    weight scales the expert's INPUT - with act(g, u) = g' sigmoid(alpha g') (u' + 1),
+    g' = min(g, limit), u' = clamp(u, -limit, limit).
+    ``glu`` "silu": out[t] = sum_j w expert_e(h_t) (+ ``addend``[t], e.g. a shared expert) - the
+    weight scales the expert's OUTPUT, in fp32 - with expert_e(x) = W_down[e] (silu(W_gate[e] x) *
+    (W_up[e] x)); an index e >= E is an identity expert, expert_e(x) = x, without weights.
+
+    On the GPU: one planning kernel sorts the (row, choice) pairs by expert into tiles of
+    MOE_TILE_ROWS (or MOE_BIG_TILE_ROWS), then two grouped matrix products (gate | up with the
+    activation in the epilogue; down) run over the tiles - no host synchronisation, so the step
+    can be captured in a graph.  Steps whose expert products reach MOE_LIBRARY_FLOPS run library
+    products per expert instead (outside a capture)."""
+    silu_glu = glu == "silu"
+    if not silu_glu and (glu != "clamped" or addend is not None):
+        raise ValueError("moe_experts: glu is 'clamped' or 'silu'; an addend goes with 'silu'")
     if not h.is_cuda:
-        return mref.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha)
+        return mref.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, silu_glu, addend)
     T, W = h.shape
     E, ff = w_gu.shape[0], w_gu.shape[1] // 2
     k = idx.shape[1]
     P = T * k
     if 0 < MOE_LIBRARY_FLOPS <= 6.0 * P * ff * W and not torch.cuda.is_current_stream_capturing():
-        return _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha)
+        return _moe_experts_library(h, idx, wts, w_gu, w_down, limit, alpha, silu_glu, addend)
     big = (h.dtype == torch.bfloat16 and W % 8 == 0 and ff % 8 == 0 and P >= MOE_BIG_TILE_PAIRS)
     rows = MOE_BIG_TILE_ROWS if big else MOE_TILE_ROWS
     max_tiles = P // rows + min(E, P)
@@ -498,5 +540,30 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702):
     act = torch.empty(P, ff, dtype=h.dtype, device=dev)
     y = torch.empty(P * split, W, dtype=torch.float32 if split > 1 else h.dtype, device=dev)
     _native().moe_experts(y, act, plan, h, idx, wts, w_gu[:, :ff], w_gu[:, ff:], w_down,
-                          float(limit), float(alpha), max_tiles, rows, split)
+                          float(limit), float(alpha), max_tiles, rows, split, int(silu_glu))
+    if silu_glu:
+        return _moe_combine(y, idx, wts, h, addend, E, split)
     return _pair_sum(y, T, k * split, h.dtype)
+
+
+def norm_add_norm(x, y, w_post, w_next, eps, kind="layer", dtype=torch.bfloat16):
+    """Layer boundary of a sandwich-norm residual in one pass: x (fp32 [T, W], in place) +=
+    norm(y) * w_post (y None: nothing is added), then returns norm(x) * w_next in ``dtype``
+    (None when ``w_next`` is None).  ``kind`` "layer": (v - mean) / sqrt(var + eps) with var the
+    mean squared deviation; "rms": v / sqrt(mean(v^2) + eps).  Sums and statistics in fp32."""
+    if kind not in ("layer", "rms"):
+        raise ValueError(kind)
+    if not x.is_cuda:
+        return mref.norm_add_norm(x, y, w_post, w_next, eps, kind == "layer", dtype)
+    h = torch.empty(x.shape, dtype=dtype, device=x.device) if w_next is not None else None
+    _native().norm_add_norm(h, x, y, w_post, w_next, eps, kind == "layer")
+    return h
+
+
+def scale_softcap(logits, scale=1.0, cap=0.0):
+    """fp32 cap * tanh(logits * scale / cap) of activation-dtype logits (cap 0: logits * scale)."""
+    if not logits.is_cuda:
+        return mref.scale_softcap(logits, float(scale), float(cap))
+    out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    _native().scale_softcap(out, logits, float(scale), float(cap))
+    return out

@@ -67,8 +67,9 @@ def rotate_interleaved(x, cos_sin):
 
 def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
                        k_cache, v_cache, heads, kv_heads, dim, vdim, rotate_half_pairs=False,
-                       norm_last=False):
-    """Per-head RMS norm (plain weight, or none when ``q_norm`` / ``k_norm`` is None) and rotary
+                       norm_last=False, whole_norm=False):
+    """Per-head RMS norm (plain weight, or none when ``q_norm`` / ``k_norm`` is None; with
+    ``whole_norm`` one norm over all heads of the projection with weights [heads * dim]) and rotary
     positions on q [T, heads * dim] and k [T, kv_heads * dim] (row-strided views); returns
     q [T, heads, dim] and writes k and v [T, kv_heads * vdim] into the paged caches
     k_cache [nb, kv_heads, BS, dim], v_cache [nb, kv_heads, vdim, BS] (channel-major pages).
@@ -81,6 +82,9 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     v = vx.reshape(T, kv_heads, vdim)
 
     def nrm(x, w):
+        if whole_norm:
+            y = x * torch.rsqrt(x.pow(2).mean((-2, -1), keepdim=True) + eps)
+            return y * w.float().view(x.shape[1], x.shape[2]) if w is not None else y
         y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
         return y * w.float() if w is not None else y
 
@@ -372,9 +376,13 @@ def token_shift(n, mu, shift_state, positions, seq_qstart, seq_slot, dtype):
 
 
 def gate_mul(a, gate, act):
-    """a [T, N] times sigmoid (act 1) or SiLU (act 0) of gate [T, N] (row-strided)."""
+    """a [T, N] times sigmoid (act 1), SiLU (act 0) or tanh-form GELU (act 2) of gate [T, N]
+    (both row-strided)."""
     g = gate.float()
-    g = torch.sigmoid(g) if act == 1 else g * torch.sigmoid(g)
+    if act == 2:
+        g = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g)))
+    else:
+        g = torch.sigmoid(g) if act == 1 else g * torch.sigmoid(g)
     return (a.float() * g).to(a.dtype)
 
 
@@ -405,20 +413,38 @@ def gelu(x, tanh_form=False):
     return F.gelu(x.float(), approximate="tanh" if tanh_form else "none").to(x.dtype)
 
 
-def moe_route(logits, top):
-    """Sigmoid scores of fp32 router logits [T, E]; the ``top`` largest per row (ties: lowest
-    index) -> (int32 [T, top], fp32 [T, top])."""
-    s = torch.sigmoid(logits.float())
-    order = torch.argsort(s, dim=1, descending=True, stable=True)[:, :top]
-    return order.to(torch.int32), torch.gather(s, 1, order)
+def moe_route(logits, top, softmax=False, correction=None, groups=1, keep=1, renorm=False):
+    """Scores (sigmoid, or softmax over the row) of fp32 router logits [T, E]; the ``top`` largest
+    per row (ties: lowest index) -> (int32 [T, top], fp32 [T, top]).  ``correction`` [E] is added
+    to the scores for the choice only; with ``groups`` > 1 only experts of the ``keep`` groups (equal
+    runs of neighbours) with the largest best choice score can be chosen; ``renorm``: the chosen
+    scores are divided by their sum + 1e-20."""
+    z = logits.float()
+    s = torch.softmax(z, 1) if softmax else torch.sigmoid(z)
+    c = s + correction.float() if correction is not None else s.clone()
+    T, E = s.shape
+    if groups > 1:
+        best = c.view(T, groups, E // groups).amax(2)
+        kept = torch.argsort(best, dim=1, descending=True, stable=True)[:, :keep]
+        allow = torch.zeros(T, groups, dtype=torch.bool, device=s.device)
+        allow.scatter_(1, kept, True)
+        c = c.masked_fill(~allow.repeat_interleave(E // groups, 1), float("-inf"))
+    order = torch.argsort(c, dim=1, descending=True, stable=True)[:, :top]
+    w = torch.gather(s, 1, order)
+    if renorm:
+        w = w / (w.sum(1, keepdim=True) + 1e-20)
+    return order.to(torch.int32), w
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha):
-    """Sum over a row's chosen experts of W_down act(W_gate (w h), W_up (w h)) with
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, silu_glu=False, addend=None):
+    """``silu_glu``: see ``moe_experts_silu``.  Otherwise:
+    sum over a row's chosen experts of W_down act(W_gate (w h), W_up (w h)) with
     act(g, u) = g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit).
     h [T, W]; idx / wts [T, k]; w_gu [E, 2 ff, W] (gate rows, then up rows); w_down [E, W, ff].
     fp32 accumulation, the activation rounded to h's dtype between the two products like the
     kernels do."""
+    if silu_glu:
+        return moe_experts_silu(h, idx, wts, w_gu, w_down, addend)
     T, W = h.shape
     out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
     hf = h.float()
@@ -428,6 +454,51 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha):
             a = clamped_glu(hf[rows] @ w_gu[e].float().T, wts[rows, j], limit, alpha).to(h.dtype)
             out[rows] += (a.float() @ w_down[e].float().T).to(h.dtype).float()
     return out.to(h.dtype)
+
+
+def moe_experts_silu(h, idx, wts, w_gu, w_down, addend=None):
+    """out[t] = sum_j w[t, j] expert_{idx[t, j]}(h_t) (+ addend[t]) with
+    expert_e(x) = W_down[e] (silu(W_gate[e] x) * (W_up[e] x)) for e < E and expert_e(x) = x for the
+    identity experts e >= E.  The weights multiply the experts' outputs in fp32; the activation
+    and each expert's output are rounded to h's dtype like the kernels do."""
+    T, W = h.shape
+    E, ff = w_gu.shape[0], w_gu.shape[1] // 2
+    out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
+    hf = h.float()
+    for j in range(idx.shape[1]):
+        for e in torch.unique(idx[:, j]).tolist():
+            rows = (idx[:, j] == e).nonzero().flatten()
+            w = wts[rows, j].float()[:, None]
+            if e >= E:
+                out[rows] += w * hf[rows]
+                continue
+            gu = hf[rows] @ w_gu[e].float().T
+            a = (gu[:, :ff] * torch.sigmoid(gu[:, :ff]) * gu[:, ff:]).to(h.dtype)
+            out[rows] += w * (a.float() @ w_down[e].float().T).to(h.dtype).float()
+    if addend is not None:
+        out += addend.float()
+    return out.to(h.dtype)
+
+
+def norm_add_norm(x, y, w_post, w_next, eps, layer, dtype):
+    """x (fp32 [T, W], in place) += norm(y) * w_post (nothing when y is None); returns
+    norm(x) * w_next in ``dtype`` (None when w_next is None).  norm: the layer norm
+    (x - mean) / sqrt(var + eps) when ``layer``, else x / sqrt(mean(x^2) + eps); all in fp32."""
+    def nrm(v, w):
+        v = v.float()
+        if layer:
+            v = v - v.mean(-1, keepdim=True)
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    if y is not None:
+        x += nrm(y, w_post)
+    return nrm(x, w_next).to(dtype) if w_next is not None else None
+
+
+def scale_softcap(logits, scale, cap):
+    """fp32 cap * tanh(logits * scale / cap) (cap 0: logits * scale)."""
+    z = logits.float() * scale
+    return cap * torch.tanh(z / cap) if cap > 0 else z
 
 
 def clamped_glu(gu, wts, limit, alpha):
