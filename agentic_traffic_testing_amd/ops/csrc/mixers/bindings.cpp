@@ -155,7 +155,8 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                         const c10::optional<at::Tensor>& k_norm, double eps,
                         const at::Tensor& positions, const at::Tensor& slot_mapping,
                         const at::Tensor& cos_sin, at::Tensor k_cache, at::Tensor v_cache,
-                        bool rotate_half, bool norm_last) {
+                        bool rotate_half, bool norm_last,
+                        const c10::optional<at::Tensor>& row_inv) {
   TORCH_CHECK(q_out.dim() == 3 && q_out.is_contiguous() && k_cache.dim() == 4 &&
                   v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "qk_norm_rope_cache: q_out [T, H, d], caches [nb, G, BS, d]");
@@ -178,11 +179,20 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                   k_cache.scalar_type() == q_out.scalar_type() &&
                   v_cache.scalar_type() == q_out.scalar_type(),
               "qk_norm_rope_cache: shapes");
-  for (const auto* w : {&q_norm, &k_norm})
+  // row_inv [T, 2]: the inverse RMS of the whole q / k projection of every row; the weights then
+  // cover the projection, [H * dim] and [G * dim]
+  if (row_inv) {
+    f32c(*row_inv, "row_inv");
+    TORCH_CHECK(row_inv->numel() == 2 * T && !norm_last, "qk_norm_rope_cache: row_inv [T, 2]");
+  }
+  int64_t heads_of = H;
+  for (const auto* w : {&q_norm, &k_norm}) {
     if (w->has_value())
-      TORCH_CHECK((*w)->is_cuda() && (*w)->numel() == dim && (*w)->is_contiguous() &&
-                      (*w)->scalar_type() == q_out.scalar_type(),
-                  "qk_norm_rope_cache: norm weights [dim]");
+      TORCH_CHECK((*w)->is_cuda() && (*w)->numel() == (row_inv ? heads_of * dim : dim) &&
+                      (*w)->is_contiguous() && (*w)->scalar_type() == q_out.scalar_type(),
+                  "qk_norm_rope_cache: norm weights [dim] (or [heads * dim] with row_inv)");
+    heads_of = G;
+  }
   const at::DeviceGuard g(qx.device());
   rc_ok(mixk_qk_norm_rope_cache(q_out.data_ptr(), qx.data_ptr(), qx.stride(0), kx.data_ptr(),
                                 kx.stride(0), vx.data_ptr(), vx.stride(0),
@@ -191,7 +201,8 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                                 positions.data_ptr<int>(), slot_mapping.data_ptr<int>(),
                                 cos_sin.data_ptr<float>(), n_freq, k_cache.data_ptr(),
                                 v_cache.data_ptr(), T, H, G, dim, vdim, BS, rotate_half, norm_last,
-                                code(q_out), cur_stream()),
+                                row_inv ? row_inv->data_ptr<float>() : nullptr, code(q_out),
+                                cur_stream()),
         "qk_norm_rope_cache");
 }
 
@@ -572,13 +583,13 @@ void token_shift(at::Tensor out, const at::Tensor& n, const at::Tensor& mu, at::
 
 void gate_mul(at::Tensor out, const at::Tensor& a, const at::Tensor& gate, int64_t act) {
   rows2d(gate, out, "gate");
-  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && a.is_cuda() && a.is_contiguous() &&
-                  a.dim() == 2 && out.sizes() == a.sizes() && gate.sizes() == a.sizes() &&
-                  a.scalar_type() == out.scalar_type(),
+  rows2d(a, out, "a");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.sizes() == a.sizes() &&
+                  gate.sizes() == a.sizes() && act >= 0 && act <= 2,
               "gate_mul: shapes");
   const at::DeviceGuard g(a.device());
-  rc_ok(mixk_gate_mul(out.data_ptr(), a.data_ptr(), gate.data_ptr(), gate.stride(0), a.size(0),
-                      a.size(1), act, code(out), cur_stream()),
+  rc_ok(mixk_gate_mul(out.data_ptr(), a.data_ptr(), a.stride(0), gate.data_ptr(), gate.stride(0),
+                      a.size(0), a.size(1), act, code(out), cur_stream()),
         "gate_mul");
 }
 
@@ -611,8 +622,19 @@ void mingru_scan(at::Tensor out, at::Tensor state, const at::Tensor& z, const at
         "mingru_scan");
 }
 
-void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits) {
+void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits, bool softmax,
+               const c10::optional<at::Tensor>& correction, int64_t groups, int64_t keep,
+               bool renorm) {
   f32c(logits, "logits");
+  if (correction) {
+    f32c(*correction, "correction");
+    TORCH_CHECK(logits.dim() == 2 && correction->numel() == logits.size(1),
+                "moe_route: correction [E]");
+  }
+  TORCH_CHECK(logits.dim() == 2 && groups >= 1 && logits.size(1) % groups == 0 && keep >= 1 &&
+                  keep <= groups && idx.dim() == 2 &&
+                  idx.size(1) <= keep * (logits.size(1) / groups),
+              "moe_route: groups must split the experts evenly and the kept ones hold `top`");
   f32c(wts, "wts");
   i32(idx, "idx");
   TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2 && idx.size(0) == logits.size(0) &&
@@ -620,14 +642,15 @@ void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits) {
               "moe_route: logits [T, E], idx / wts [T, top]");
   const at::DeviceGuard g(logits.device());
   rc_ok(mixk_moe_route(idx.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(),
-                       logits.size(0), logits.size(1), idx.size(1), cur_stream()),
+                       correction ? correction->data_ptr<float>() : nullptr, logits.size(0),
+                       logits.size(1), idx.size(1), softmax, groups, keep, renorm, cur_stream()),
         "moe_route");
 }
 
 void moe_experts(at::Tensor y, at::Tensor act, at::Tensor plan, const at::Tensor& h,
                  const at::Tensor& idx, const at::Tensor& wts, const at::Tensor& w_gate,
                  const at::Tensor& w_up, const at::Tensor& w_down, double limit, double alpha,
-                 int64_t max_tiles, int64_t tile_rows, int64_t split) {
+                 int64_t max_tiles, int64_t tile_rows, int64_t split, int64_t glu) {
   i32(idx, "idx");
   i32(plan, "plan");
   f32c(wts, "wts");
@@ -655,7 +678,7 @@ void moe_experts(at::Tensor y, at::Tensor act, at::Tensor plan, const at::Tensor
                          idx.data_ptr<int>(), wts.data_ptr<float>(), w_gate.data_ptr(),
                          w_up.data_ptr(), w_down.data_ptr(), T, top, E, ff, W, w_gate.stride(0), max_tiles,
                          tile_rows, split,
-                         static_cast<float>(limit), static_cast<float>(alpha), code(h),
+                         static_cast<float>(limit), static_cast<float>(alpha), glu, code(h),
                          cur_stream()),
         "moe_experts");
 }
@@ -687,6 +710,85 @@ void clamped_glu(at::Tensor out, const at::Tensor& gu, const at::Tensor& wts, do
         "clamped_glu");
 }
 
+void moe_combine(at::Tensor out, const at::Tensor& y, const at::Tensor& idx, const at::Tensor& wts,
+                 const at::Tensor& h, const c10::optional<at::Tensor>& addend, int64_t E,
+                 int64_t split) {
+  i32(idx, "idx");
+  f32c(wts, "wts");
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous() && out.is_cuda() &&
+                  out.is_contiguous() && out.sizes() == h.sizes() &&
+                  out.scalar_type() == h.scalar_type() && idx.dim() == 2 &&
+                  idx.size(0) == h.size(0) && wts.sizes() == idx.sizes() && split >= 1 &&
+                  y.is_cuda() && y.is_contiguous() && y.dim() == 2 &&
+                  y.size(0) == h.size(0) * idx.size(1) * split && y.size(1) == h.size(1) &&
+                  (y.scalar_type() == h.scalar_type() || y.scalar_type() == at::kFloat) && E >= 0,
+              "moe_combine: h / out [T, W], idx / wts [T, top], y [T * top * split, W]");
+  if (addend)
+    TORCH_CHECK(addend->is_cuda() && addend->is_contiguous() && addend->sizes() == h.sizes() &&
+                    addend->scalar_type() == h.scalar_type(),
+                "moe_combine: addend [T, W]");
+  const at::DeviceGuard g(h.device());
+  rc_ok(mixk_moe_combine(out.data_ptr(), y.data_ptr(), y.scalar_type() == at::kFloat,
+                         idx.data_ptr<int>(), wts.data_ptr<float>(), h.data_ptr(),
+                         addend ? addend->data_ptr() : nullptr, h.size(0), idx.size(1), split, E,
+                         h.size(1), code(h), cur_stream()),
+        "moe_combine");
+}
+
+void norm_add_norm(const c10::optional<at::Tensor>& h, at::Tensor x,
+                   const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& w_post,
+                   const c10::optional<at::Tensor>& w_next, double eps, bool layer) {
+  f32c(x, "x");
+  TORCH_CHECK(x.dim() == 2 && (h.has_value() || y.has_value()) &&
+                  h.has_value() == w_next.has_value() && y.has_value() == w_post.has_value(),
+              "norm_add_norm: x [T, W]; y with w_post, h with w_next");
+  const at::Tensor& like = h ? *h : *y;
+  auto rows = [&](const at::Tensor& t) {
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.sizes() == x.sizes() &&
+                    t.scalar_type() == like.scalar_type(),
+                "norm_add_norm: rows [T, W] of one activation dtype");
+  };
+  auto weight = [&](const at::Tensor& t) {
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.numel() == x.size(1) &&
+                    t.scalar_type() == like.scalar_type(),
+                "norm_add_norm: weights [W] of the activation dtype");
+  };
+  if (h) { rows(*h); weight(*w_next); }
+  if (y) { rows(*y); weight(*w_post); }
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_norm_add_norm(h ? h->data_ptr() : nullptr, x.data_ptr<float>(),
+                           y ? y->data_ptr() : nullptr, w_post ? w_post->data_ptr() : nullptr,
+                           w_next ? w_next->data_ptr() : nullptr, x.size(0), x.size(1),
+                           static_cast<float>(eps), layer, code(like), cur_stream()),
+        "norm_add_norm");
+}
+
+void proj_inv_rms(at::Tensor out, const at::Tensor& qx, const at::Tensor& kx, double eps) {
+  f32c(out, "out");
+  rows2d(qx, qx, "q");
+  rows2d(kx, qx, "k");
+  TORCH_CHECK(out.numel() == 2 * qx.size(0) && kx.size(0) == qx.size(0) && qx.size(1) > 0 &&
+                  kx.size(1) > 0,
+              "proj_inv_rms: out [T, 2], q [T, nq], k [T, nk]");
+  const at::DeviceGuard g(qx.device());
+  rc_ok(mixk_proj_inv_rms(out.data_ptr<float>(), qx.data_ptr(), qx.stride(0), qx.size(1),
+                          kx.data_ptr(), kx.stride(0), kx.size(1), qx.size(0),
+                          static_cast<float>(eps), code(qx), cur_stream()),
+        "proj_inv_rms");
+}
+
+void scale_softcap(at::Tensor out, const at::Tensor& logits, double scale, double cap) {
+  f32c(out, "out");
+  TORCH_CHECK(logits.is_cuda() && logits.is_contiguous() && out.sizes() == logits.sizes() &&
+                  cap >= 0.0,
+              "scale_softcap: contiguous logits, fp32 out of the same shape");
+  const at::DeviceGuard g(logits.device());
+  rc_ok(mixk_scale_softcap(out.data_ptr<float>(), logits.data_ptr(), logits.numel(),
+                           static_cast<float>(scale), static_cast<float>(cap), code(logits),
+                           cur_stream()),
+        "scale_softcap");
+}
+
 }  // namespace
 
 TORCH_LIBRARY(atta_mix, m) {
@@ -701,7 +803,8 @@ TORCH_LIBRARY(atta_mix, m) {
   m.def("gated_rms_norm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, float eps, int act) -> ()");
   m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor? q_norm, "
         "Tensor? k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor cos_sin, "
-        "Tensor(b!) k_cache, Tensor(c!) v_cache, bool rotate_half, bool norm_last) -> ()");
+        "Tensor(b!) k_cache, Tensor(c!) v_cache, bool rotate_half, bool norm_last, "
+        "Tensor? row_inv) -> ()");
   m.def("rotary_table(Tensor(a!) out, Tensor positions, Tensor inv_freq) -> ()");
   m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
@@ -734,10 +837,17 @@ TORCH_LIBRARY(atta_mix, m) {
         "Tensor positions, Tensor seq_qstart, Tensor seq_slot) -> ()");
   m.def("pair_sum(Tensor(a!) out, Tensor y) -> ()");
   m.def("clamped_glu(Tensor(a!) out, Tensor gu, Tensor wts, float limit, float alpha) -> ()");
-  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits) -> ()");
+  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, bool softmax, Tensor? correction, "
+        "int groups, int keep, bool renorm) -> ()");
   m.def("moe_experts(Tensor(a!) y, Tensor(b!) act, Tensor(c!) plan, Tensor h, Tensor idx, "
         "Tensor wts, Tensor w_gate, Tensor w_up, Tensor w_down, float limit, float alpha, "
-        "int max_tiles, int tile_rows, int split) -> ()");
+        "int max_tiles, int tile_rows, int split, int glu) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor idx, Tensor wts, Tensor h, Tensor? addend, "
+        "int E, int split) -> ()");
+  m.def("norm_add_norm(Tensor(a!)? h, Tensor(b!) x, Tensor? y, Tensor? w_post, Tensor? w_next, "
+        "float eps, bool layer) -> ()");
+  m.def("proj_inv_rms(Tensor(a!) out, Tensor qx, Tensor kx, float eps) -> ()");
+  m.def("scale_softcap(Tensor(a!) out, Tensor logits, float scale, float cap) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
@@ -768,4 +878,8 @@ TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
   m.impl("clamped_glu", &clamped_glu);
   m.impl("moe_route", &moe_route);
   m.impl("moe_experts", &moe_experts);
+  m.impl("moe_combine", &moe_combine);
+  m.impl("norm_add_norm", &norm_add_norm);
+  m.impl("proj_inv_rms", &proj_inv_rms);
+  m.impl("scale_softcap", &scale_softcap);
 }

@@ -233,35 +233,39 @@ __global__ void token_shift_kernel(T* __restrict__ out, const float* __restrict_
   }
 }
 
+__device__ __forceinline__ float gelu_(float z, bool tanh_form) {
+  if (tanh_form)
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+}
+
+// act: 0 SiLU, 1 sigmoid, 2 tanh-form GELU
+__device__ __forceinline__ float gate_act(float g, int act) {
+  return act == 1 ? sigmoidf_(g) : act == 2 ? gelu_(g, true) : siluf_(g);
+}
+
 template <typename T>
-__global__ void gate_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
+__global__ void gate_mul_kernel(T* __restrict__ out, const T* __restrict__ a, int64_t a_stride,
                                 const T* __restrict__ gate, int64_t gate_stride, int N, int act) {
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= N) return;
   const float g = ldf(gate + blockIdx.x * gate_stride + i);
-  const int64_t o = static_cast<int64_t>(blockIdx.x) * N + i;
-  stf(out + o, ldf(a + o) * (act == 1 ? sigmoidf_(g) : siluf_(g)));
+  stf(out + static_cast<int64_t>(blockIdx.x) * N + i,
+      ldf(a + blockIdx.x * a_stride + i) * gate_act(g, act));
 }
 
 template <typename T>
-__global__ void gate_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ a,
+__global__ void gate_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ a, int64_t a_stride,
                                     const T* __restrict__ gate, int64_t gate_stride, int N,
                                     int act) {
   const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (i >= N) return;
   float g[8], v[8];
   ld8(gate + blockIdx.x * gate_stride + i, g);
-  const int64_t o = static_cast<int64_t>(blockIdx.x) * N + i;
-  ld8(a + o, v);
+  ld8(a + blockIdx.x * a_stride + i, v);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) v[e] *= act == 1 ? sigmoidf_(g[e]) : siluf_(g[e]);
-  st8(out + o, v);
-}
-
-__device__ __forceinline__ float gelu_(float z, bool tanh_form) {
-  if (tanh_form)
-    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-  return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+  for (int e = 0; e < 8; ++e) v[e] *= gate_act(g[e], act);
+  st8(out + static_cast<int64_t>(blockIdx.x) * N + i, v);
 }
 
 template <typename T>
@@ -421,19 +425,21 @@ extern "C" int mixk_token_shift(void* out, const float* n, const float* mu, floa
   return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int mixk_gate_mul(void* out, const void* a, const void* gate, int64_t gate_stride,
-                             int T_, int N, int act, int dtype, hipStream_t st) {
+extern "C" int mixk_gate_mul(void* out, const void* a, int64_t a_stride, const void* gate,
+                             int64_t gate_stride, int T_, int N, int act, int dtype,
+                             hipStream_t st) {
   if (T_ <= 0 || N <= 0) return 0;
-  const bool vec = N % 8 == 0 && gate_stride % 8 == 0 && aligned16(out) && aligned16(a) &&
-                   aligned16(gate);
+  if (act < 0 || act > 2) return -1;
+  const bool vec = N % 8 == 0 && gate_stride % 8 == 0 && a_stride % 8 == 0 && aligned16(out) &&
+                   aligned16(a) && aligned16(gate);
   MIXK_DISPATCH(dtype, {
     if (vec)
       hipLaunchKernelGGL(gate_mul_vec_kernel<T>, dim3(T_, (N / 8 + 255) / 256), dim3(256), 0, st,
-                         static_cast<T*>(out), static_cast<const T*>(a),
+                         static_cast<T*>(out), static_cast<const T*>(a), a_stride,
                          static_cast<const T*>(gate), gate_stride, N, act);
     else
       hipLaunchKernelGGL(gate_mul_kernel<T>, dim3(T_, (N + 255) / 256), dim3(256), 0, st,
-                         static_cast<T*>(out), static_cast<const T*>(a),
+                         static_cast<T*>(out), static_cast<const T*>(a), a_stride,
                          static_cast<const T*>(gate), gate_stride, N, act);
   });
   return static_cast<int>(hipGetLastError());

@@ -26,7 +26,8 @@ int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_stride, const
                             const void* k_norm, float eps, const int* positions,
                             const int* slot_mapping, const float* cos_sin, int n_freq,
                             void* k_cache, void* v_cache, int T, int H, int G, int dim, int vdim,
-                            int block_size, int half, int norm_last, int dtype, hipStream_t st);
+                            int block_size, int half, int norm_last, const float* row_inv,
+                            int dtype, hipStream_t st);
 int mixk_rotary_table(float* out, const int* positions, const float* inv_freq, int T, int n_freq,
                       hipStream_t st);
 int mixk_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -73,8 +74,8 @@ int mixk_hyper_update_norm(void* out, int out_f32, float* xs, const void* y, con
 int mixk_token_shift(void* out, const float* n, const float* mu, float* state,
                      const int* positions, const int* seq_qstart, const int* seq_slot, int T,
                      int S, int W, int dtype, hipStream_t st);
-int mixk_gate_mul(void* out, const void* a, const void* gate, int64_t gate_stride, int T, int N,
-                  int act, int dtype, hipStream_t st);
+int mixk_gate_mul(void* out, const void* a, int64_t a_stride, const void* gate,
+                  int64_t gate_stride, int T, int N, int act, int dtype, hipStream_t st);
 int mixk_gelu(void* out, const void* x, int64_t x_stride, int T, int N, int tanh_form, int dtype,
               hipStream_t st);
 int mixk_mingru_scan(void* out, float* state, const void* z, int64_t z_stride, const void* x,
@@ -85,11 +86,20 @@ int mixk_clamped_glu(void* out, const void* gu, const float* wts, int R, int ff,
                      float alpha, int dtype, hipStream_t st);
 int mixk_pair_sum(void* out, const void* y, int y_f32, int T, int top, int W, int dtype,
                   hipStream_t st);
-int mixk_moe_route(int* idx, float* wts, const float* logits, int T, int E, int top,
-                   hipStream_t st);
+int mixk_moe_route(int* idx, float* wts, const float* logits, const float* correction, int T,
+                   int E, int top, int softmax, int groups, int keep, int renorm, hipStream_t st);
 int mixk_moe_experts(void* y, void* act, int* plan, const void* h, const int* idx,
                      const float* wts, const void* w_gate, const void* w_up, const void* w_down,
                      int T, int top, int E, int ff, int W, int64_t gu_estride, int max_tiles,
                      int tile_rows, int split, float limit,
-                     float alpha, int dtype, hipStream_t st);
+                     float alpha, int glu, int dtype, hipStream_t st);
+int mixk_moe_combine(void* out, const void* y, int y_f32, const int* idx, const float* wts,
+                     const void* h, const void* addend, int T, int top, int split, int E, int W,
+                     int dtype, hipStream_t st);
+int mixk_norm_add_norm(void* h, float* x, const void* y, const void* w_post, const void* w_next,
+                       int T, int W, float eps, int layer, int dtype, hipStream_t st);
+int mixk_proj_inv_rms(float* out, const void* qx, int64_t q_stride, int nq, const void* kx,
+                      int64_t k_stride, int nk, int T, float eps, int dtype, hipStream_t st);
+int mixk_scale_softcap(float* out, const void* x, int64_t n, float scale, float cap, int dtype,
+                       hipStream_t st);
 }

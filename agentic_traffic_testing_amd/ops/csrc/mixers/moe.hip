@@ -1,9 +1,14 @@
-// Routed experts: sigmoid top-k routing, an on-device plan that sorts the (row, choice) pairs by
+// Routed experts: top-k routing (sigmoid or softmax scores, optional choice correction and
+// group-limited choice, optional renormalisation), an on-device plan that sorts the (row, choice) pairs by
 // expert into tiles, and grouped matrix products over the tiles - no host round trip, so a step
 // can be recorded in a graph.
 //
-// * moe_route: one wave per row of fp32 router logits [T, E]; scores = sigmoid; `top` rounds of
-//   wave-wide arg-max (ties: lowest index) give idx [T, top] and the scores wts [T, top].
+// * moe_route: one wave per row of fp32 router logits [T, E]; scores = sigmoid, or softmax over
+//   the row; choice scores = scores (+ correction[e]); with groups > 1 a group (E / groups
+//   neighbouring experts) scores its largest choice score, `keep` rounds of wave-wide arg-max
+//   pick the groups whose experts stay eligible; `top` rounds of wave-wide arg-max over the
+//   eligible choice scores (ties: lowest index) give idx [T, top]; wts [T, top] are the plain
+//   scores of the chosen, optionally divided by their sum + 1e-20.
 // * moe_plan (one workgroup): histogram of the P = T * top pairs over the experts, prefix sums,
 //   the tile table (expert, first sorted position, rows <= rows_per_tile), and the pairs scattered
 //   into expert order.  plan = [ntiles, 0, tile_expert[max_tiles], tile_start[max_tiles],
@@ -26,8 +31,11 @@
 //   (four 32 x 32 blocks per wave) in the plain form and 128 rows x 64 features of gate and of
 //   up in the GLU form (the same four blocks per wave and LDS per workgroup).  Rows kernel (any dtype and sizes): fp32 FMA, 4 x 4 outputs per thread from fp32
 //   LDS tiles of 64 rows x 64 features.
+//   With glu = 1 the first product's epilogue is the plain SiLU GLU, silu(acc_g) acc_u, without
+//   the router weight (moe_combine applies it to the expert's output).
 // * clamped_glu (rows of [gate | up] products from library GEMMs), pair_sum (a row's choices and
-//   split partials added in fp32).
+//   split partials added in fp32), moe_combine (out[t] = sum_j w[t, j] y[t, j] (+ addend[t]) in
+//   fp32, where an index >= E is an identity expert whose output is the row of h itself).
 #include "mix_common.h"
 #include "mixers.h"
 
@@ -38,45 +46,139 @@ constexpr int kMoeFeat = 64;        // output features per workgroup
 constexpr int kMaxExperts = 1024;
 constexpr int kRoutePer = kMaxExperts / kWave;
 
-__global__ void moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts,
-                                 const float* __restrict__ logits, int T_, int E, int top) {
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (t >= T_) return;
+__device__ __forceinline__ void wave_argmax(float& best, int& be) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, kWave);
+    const int oe = __shfl_xor(be, o, kWave);
+    if (ob > best || (ob == best && oe < be)) {
+      best = ob;
+      be = oe;
+    }
+  }
+}
+
+// Every wave runs to the end (rows past T_ recompute the last row and write nothing), so the
+// workgroup barriers around the LDS exchange of the grouped form are reached by all of them.
+__global__ void __launch_bounds__(256)
+moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
+                 const float* __restrict__ correction, int T_, int E, int top, int softmax,
+                 int groups, int keep, int renorm) {
+  __shared__ float s_choice[4][kMaxExperts];
+  __shared__ unsigned char s_kept[4][kMaxExperts];
+  const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t_raw = blockIdx.x * 4 + wv;
+  const bool live = t_raw < T_;
+  const int t = live ? t_raw : T_ - 1;
   const float* row = logits + static_cast<int64_t>(t) * E;
-  float sc[kRoutePer];
+  float sc[kRoutePer], ch[kRoutePer];
+  int pick[kRoutePer];
+  float zmax = -INFINITY;
 #pragma unroll
   for (int j = 0; j < kRoutePer; ++j) {
     const int e = lane + j * kWave;
-    sc[j] = e < E ? sigmoidf_(row[e]) : -1.f;   // scores lie in [0, 1]
+    sc[j] = e < E ? row[e] : -INFINITY;
+    zmax = fmaxf(zmax, sc[j]);
+    pick[j] = -1;
   }
-  for (int k = 0; k < top; ++k) {
-    float best = -2.f;
-    int be = 0x7fffffff;
+  if (softmax) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) zmax = fmaxf(zmax, __shfl_xor(zmax, o, kWave));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) {
+      sc[j] = lane + j * kWave < E ? expf(sc[j] - zmax) : 0.f;
+      sum += sc[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) sc[j] = sc[j] / sum;
+  } else {
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) sc[j] = sigmoidf_(sc[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < kRoutePer; ++j) {
+    const int e = lane + j * kWave;
+    ch[j] = e < E ? sc[j] + (correction != nullptr ? correction[e] : 0.f) : -INFINITY;
+  }
+  if (groups > 1) {   // uniform over the launch
+    const int gs = E / groups;
 #pragma unroll
     for (int j = 0; j < kRoutePer; ++j) {
       const int e = lane + j * kWave;
-      if (sc[j] > best) {   // ascending e inside a lane: the first of equals wins
-        best = sc[j];
-        be = e;
-      }
+      if (e < E) s_choice[wv][e] = ch[j];
+      if (e < groups) s_kept[wv][e] = 0;
     }
+    __syncthreads();
+    float gm[kRoutePer];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ob = __shfl_xor(best, o, kWave);
-      const int oe = __shfl_xor(be, o, kWave);
-      if (ob > best || (ob == best && oe < be)) {
-        best = ob;
-        be = oe;
-      }
+    for (int j = 0; j < kRoutePer; ++j) {
+      const int g = lane + j * kWave;
+      gm[j] = -INFINITY;
+      if (g < groups)
+        for (int i = 0; i < gs; ++i) gm[j] = fmaxf(gm[j], s_choice[wv][g * gs + i]);
     }
-    if (lane == 0) {
-      idx[static_cast<int64_t>(t) * top + k] = be;
-      wts[static_cast<int64_t>(t) * top + k] = best;
+    for (int k = 0; k < keep; ++k) {
+      float best = -INFINITY;
+      int be = 0x7fffffff;
+#pragma unroll
+      for (int j = 0; j < kRoutePer; ++j)
+        if (gm[j] > best) {
+          best = gm[j];
+          be = lane + j * kWave;
+        }
+      wave_argmax(best, be);
+#pragma unroll
+      for (int j = 0; j < kRoutePer; ++j)
+        if (lane + j * kWave == be) {
+          gm[j] = -INFINITY;
+          s_kept[wv][be] = 1;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) {
+      const int e = lane + j * kWave;
+      if (e < E && !s_kept[wv][e / gs]) ch[j] = -INFINITY;
+    }
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j)
+      if (ch[j] > best) {   // ascending e inside a lane: the first of equals wins
+        best = ch[j];
+        be = lane + j * kWave;
+      }
+    wave_argmax(best, be);
+    if (be == 0x7fffffff) {   // nothing eligible is left (non-finite scores): a zero weight
+      if (live && lane == 0) {
+        idx[static_cast<int64_t>(t) * top + k] = 0;
+        wts[static_cast<int64_t>(t) * top + k] = 0.f;
+      }
+      continue;
     }
 #pragma unroll
     for (int j = 0; j < kRoutePer; ++j)
-      if (lane + j * kWave == be) sc[j] = -1.f;
+      if (lane + j * kWave == be) {
+        ch[j] = -INFINITY;
+        pick[j] = k;
+      }
   }
+  float tot = 0.f;
+#pragma unroll
+  for (int j = 0; j < kRoutePer; ++j)
+    if (pick[j] >= 0) tot += sc[j];
+  tot = wave_sum(tot);
+  if (!live) return;
+#pragma unroll
+  for (int j = 0; j < kRoutePer; ++j)
+    if (pick[j] >= 0) {
+      idx[static_cast<int64_t>(t) * top + pick[j]] = lane + j * kWave;
+      wts[static_cast<int64_t>(t) * top + pick[j]] = renorm ? sc[j] / (tot + 1e-20f) : sc[j];
+    }
 }
 
 __global__ void __launch_bounds__(1024)
@@ -122,6 +224,7 @@ struct MoeArgs {
   int64_t x_stride;
   int64_t w_estride;   // elements between two experts' matrices
   float limit, alpha;
+  int glu;             // GLU form: 0 clamped GLU of the weighted products, 1 silu(g) u, no weight
   int split, k_chunk;  // plain form: blockIdx.z takes K range [z k_chunk, (z + 1) k_chunk) and
                        // writes its fp32 partial to row pair * split + z
 };
@@ -130,6 +233,10 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float wt, float l
   g = fminf(g * wt, limit);
   u = fminf(fmaxf(u * wt, -limit), limit);
   return g * sigmoidf_(alpha * g) * (u + 1.0f);
+}
+
+__device__ __forceinline__ float glu_act(float g, float u, float wt, const MoeArgs& a) {
+  return a.glu == 1 ? siluf_(g) * u : clamped_glu(g, u, wt, a.limit, a.alpha);
 }
 
 typedef __attribute__((ext_vector_type(8))) __bf16 mbf16x8;
@@ -276,8 +383,8 @@ moe_gemm_mfma_kernel(OutT* __restrict__ out, const __bf16* __restrict__ x,
         float v[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          v[q] = GLU ? clamped_glu(acc1[i][j][4 * i4 + q], acc2[GLU ? i : 0][GLU ? j : 0][4 * i4 + q],
-                                   wt, a.limit, a.alpha)
+          v[q] = GLU ? glu_act(acc1[i][j][4 * i4 + q], acc2[GLU ? i : 0][GLU ? j : 0][4 * i4 + q],
+                               wt, a)
                      : acc1[i][j][4 * i4 + q];
         if (f + 3 < N && (N & 3) == 0) {
           st4(orow + f, v);
@@ -360,7 +467,7 @@ moe_gemm_rows_kernel(T* __restrict__ out, const T* __restrict__ x, const T* __re
     for (int j = 0; j < 4; ++j) {
       const int f = f0 + tc + 16 * j;
       if (f < N)
-        stf(orow + f, GLU ? clamped_glu(acc1[i][j], acc2[i][j], wt, a.limit, a.alpha) : acc1[i][j]);
+        stf(orow + f, GLU ? glu_act(acc1[i][j], acc2[i][j], wt, a) : acc1[i][j]);
     }
   }
 }
@@ -404,9 +511,80 @@ __global__ void pair_sum_vec_kernel(T* __restrict__ out, const TI* __restrict__ 
   st8(out + static_cast<int64_t>(blockIdx.x) * W + i, a);
 }
 
+// out[t] = sum_j wts[t, j] * v_j (+ addend[t]) in fp32, j in order; v_j = the sum of the pair's
+// `split` adjacent rows of y, or the row of h when idx[t, j] >= E (an identity expert).
+template <typename T, typename TY, bool VEC>
+__global__ void moe_combine_kernel(T* __restrict__ out, const TY* __restrict__ y,
+                                   const int* __restrict__ idx, const float* __restrict__ wts,
+                                   const T* __restrict__ h, const T* __restrict__ addend, int top,
+                                   int split, int E, int W) {
+  constexpr int N = VEC ? 8 : 1;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * N;
+  if (i >= W) return;
+  const int64_t t = blockIdx.x;
+  float acc[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) acc[e] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int ex = idx[t * top + j];
+    const float w = wts[t * top + j];
+    float v[N];
+    if (ex >= E) {
+      if (VEC) ld8(h + t * W + i, v); else v[0] = ldf(h + t * W + i);
+    } else {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = 0.f;
+      const TY* src = y + (t * top + j) * split * W + i;
+      for (int z = 0; z < split; ++z) {
+        float u[N];
+        if (VEC) ld8(src + static_cast<int64_t>(z) * W, u); else u[0] = ldf(src + static_cast<int64_t>(z) * W);
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] += u[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] += w * v[e];
+  }
+  if (addend != nullptr) {
+    float u[N];
+    if (VEC) ld8(addend + t * W + i, u); else u[0] = ldf(addend + t * W + i);
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] += u[e];
+  }
+  if (VEC) st8(out + t * W + i, acc); else stf(out + t * W + i, acc[0]);
+}
+
 }  // namespace mixk
 
 using namespace mixk;
+
+extern "C" int mixk_moe_combine(void* out, const void* y, int y_f32, const int* idx,
+                                const float* wts, const void* h, const void* addend, int T_,
+                                int top, int split, int E, int W, int dtype, hipStream_t st) {
+  if (T_ <= 0 || W <= 0) return 0;
+  if (top < 1 || split < 1) return -1;
+  auto al = [](const void* p, uintptr_t m) { return (reinterpret_cast<uintptr_t>(p) & m) == 0; };
+  const uintptr_t am = dtype == 2 ? 31 : 15;
+  const bool vec = W % 8 == 0 && al(out, am) && al(h, am) && al(y, y_f32 ? 31 : am) &&
+                   (addend == nullptr || al(addend, am));
+  const dim3 grid(T_, vec ? (W / 8 + 127) / 128 : (W + 255) / 256), block(vec ? 128 : 256);
+#define MIXK_COMBINE(TY, VEC)                                                                     \
+  hipLaunchKernelGGL((moe_combine_kernel<T, TY, VEC>), grid, block, 0, st, static_cast<T*>(out),  \
+                     static_cast<const TY*>(y), idx, wts, static_cast<const T*>(h),               \
+                     static_cast<const T*>(addend), top, split, E, W)
+  MIXK_DISPATCH(dtype, {
+    if (y_f32 && vec)
+      MIXK_COMBINE(float, true);
+    else if (y_f32)
+      MIXK_COMBINE(float, false);
+    else if (vec)
+      MIXK_COMBINE(T, true);
+    else
+      MIXK_COMBINE(T, false);
+  });
+#undef MIXK_COMBINE
+  return static_cast<int>(hipGetLastError());
+}
 
 // y_f32: the summands are fp32 (split-K partials) whatever the output dtype.
 extern "C" int mixk_pair_sum(void* out, const void* y, int y_f32, int T_, int top, int W,
@@ -441,12 +619,15 @@ extern "C" int mixk_clamped_glu(void* out, const void* gu, const float* wts, int
   return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int mixk_moe_route(int* idx, float* wts, const float* logits, int T_, int E, int top,
-                              hipStream_t st) {
+extern "C" int mixk_moe_route(int* idx, float* wts, const float* logits, const float* correction,
+                              int T_, int E, int top, int softmax, int groups, int keep,
+                              int renorm, hipStream_t st) {
   if (T_ <= 0) return 0;
-  if (E < 1 || E > kMaxExperts || top < 1 || top > E) return -1;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T_ + 3) / 4), dim3(256), 0, st, idx, wts, logits, T_,
-                     E, top);
+  if (E < 1 || E > kMaxExperts || top < 1 || top > E || groups < 1 || E % groups != 0 ||
+      keep < 1 || keep > groups || top > keep * (E / groups))
+    return -1;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T_ + 3) / 4), dim3(256), 0, st, idx, wts, logits,
+                     correction, T_, E, top, softmax, groups, keep, renorm);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -458,8 +639,9 @@ extern "C" int mixk_moe_experts(void* y, void* act, int* plan, const void* h, co
                                 const float* wts, const void* w_gate, const void* w_up,
                                 const void* w_down, int T_, int top, int E, int ff, int W,
                                 int64_t gu_estride, int max_tiles, int tile_rows, int split,
-                                float limit, float alpha, int dtype, hipStream_t st) {
+                                float limit, float alpha, int glu, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
+  if (glu != 0 && glu != 1) return -1;
   const int P = T_ * top;
   const bool mfma = dtype == 0 && W % 8 == 0 && ff % 8 == 0;
   if (E < 1 || E > kMaxExperts || (tile_rows != 64 && !(tile_rows == 128 && mfma)) ||
@@ -469,11 +651,11 @@ extern "C" int mixk_moe_experts(void* y, void* act, int* plan, const void* h, co
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, st, plan, idx, P, E, max_tiles,
                      tile_rows);
   MoeArgs a1{plan, wts, max_tiles, top, ff, W, static_cast<int64_t>(W), gu_estride, limit, alpha,
-             1, W};
+             glu, 1, W};
   // the down product's K range per workgroup: a multiple of the staged K step
   const int k_chunk = split > 1 ? ((ff + split - 1) / split + kMoeBK - 1) / kMoeBK * kMoeBK : ff;
   MoeArgs a2{plan, wts, max_tiles, top, W, ff, static_cast<int64_t>(ff),
-             static_cast<int64_t>(W) * ff, limit, alpha, split, k_chunk};
+             static_cast<int64_t>(W) * ff, limit, alpha, glu, split, k_chunk};
   // feature blocks: 64 for the gate | up form (two weight tiles per block), 128 for the down form
   // of the large tiles
   const int ft2 = tile_rows == 128 && mfma ? 128 : kMoeFeat;

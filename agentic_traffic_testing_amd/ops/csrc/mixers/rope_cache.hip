@@ -1,4 +1,5 @@
-// Per-head q / k RMS norm (plain weight or none), rotary positions on the first 2 * n_freq
+// Per-head q / k RMS norm (plain weight or none; or a norm over the whole projection whose
+// per-row inverse RMS is given), rotary positions on the first 2 * n_freq
 // channels (pairs (2i, 2i + 1), or (i, i + n_freq) in the rotate-half layout; the norm before or
 // after the rotation), and the paged K / V write of the softmax mixer; further down, the front
 // end of latent attention (absorbed query assembly, rotate-half positions, latent K / V write).
@@ -38,14 +39,17 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                                           const float* __restrict__ cos_sin, int n_freq,
                                           T* __restrict__ k_cache, T* __restrict__ v_cache, int H,
                                           int G, int dim, int vdim, int block_size, int half,
-                                          int norm_last) {
+                                          int norm_last, const float* __restrict__ row_inv) {
   const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (head >= H + G) return;
   const int slot = slot_mapping[t];
   const bool is_q = head < H;
   if (!is_q && slot < 0) return;
   const T* src = is_q ? qx + t * q_stride + head * dim : kx + t * k_stride + (head - H) * dim;
+  // row_inv [T, 2]: the norm runs over the whole q (k) projection - its inverse RMS was computed
+  // per row beforehand and the weights are indexed by the projection's channel
   const T* w = is_q ? q_norm : k_norm;
+  if (row_inv != nullptr && w != nullptr) w += (is_q ? head : head - H) * dim;
   T* dst = is_q ? q_out + (static_cast<int64_t>(t) * H + head) * dim
                 : k_cache + ((static_cast<int64_t>(slot / block_size) * G + (head - H)) *
                                  block_size + slot % block_size) * dim;
@@ -71,8 +75,13 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
       ss += u[j] * u[j] + v[j] * v[j];
     }
   }
-  ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dim) + eps);
+  float inv;
+  if (row_inv != nullptr) {
+    inv = row_inv[2 * static_cast<int64_t>(t) + (is_q ? 0 : 1)];
+  } else {
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / static_cast<float>(dim) + eps);
+  }
 #pragma unroll
   for (int j = 0; j < kMaxPairs; ++j) {
     const int i = lane + j * kWave;
@@ -201,10 +210,10 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                        float eps, const int* positions, const int* slot_mapping,
                                        const float* cos_sin, int n_freq, void* k_cache,
                                        void* v_cache, int T_, int H, int G, int dim, int vdim,
-                                       int block_size, int half, int norm_last, int dtype,
-                                       hipStream_t st) {
+                                       int block_size, int half, int norm_last,
+                                       const float* row_inv, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
-  if (dim > 2 * kWave * kMaxPairs || (dim & 1)) return -1;
+  if (dim > 2 * kWave * kMaxPairs || (dim & 1) || (row_inv != nullptr && norm_last)) return -1;
   MIXK_DISPATCH(dtype,
                 hipLaunchKernelGGL(v_cache_write_kernel<T>, dim3((T_ + 7) / 8, G), dim3(128), 0,
                                    st, static_cast<const T*>(vx), v_stride, slot_mapping,
@@ -217,7 +226,7 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                    static_cast<const T*>(q_norm), static_cast<const T*>(k_norm),
                                    eps, positions, slot_mapping, cos_sin, n_freq,
                                    static_cast<T*>(k_cache), static_cast<T*>(v_cache), H, G, dim,
-                                   vdim, block_size, half, norm_last));
+                                   vdim, block_size, half, norm_last, row_inv));
   return static_cast<int>(hipGetLastError());
 }
 
