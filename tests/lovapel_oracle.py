@@ -88,7 +88,9 @@ def route(z, correction, top, groups, keep):
     """One token's router logits z [N] -> (chosen indices, their weights).  The softmax scores
     plus ``correction`` decide the choice, inside the ``keep`` groups (of ``groups`` equal runs
     of neighbours) whose best such score is largest; the weights are the plain scores of the
-    chosen, normalised to sum 1."""
+    chosen, normalised to sum 1.  Also returns how far the choice is from another one: the gap
+    between the last chosen and the best unchosen score, or between the last kept and the best
+    dropped group if that is smaller."""
     s = torch.softmax(z, 0)
     c = s + correction
     n = z.shape[0]
@@ -100,7 +102,12 @@ def route(z, correction, top, groups, keep):
         masked[g * size:(g + 1) * size] = c[g * size:(g + 1) * size]
     idx = torch.topk(masked, top).indices
     w = s[idx]
-    return idx, w / (w.sum() + 1e-20), masked
+    srt = torch.sort(masked, descending=True).values
+    margin = float(srt[top - 1] - srt[top]) if n > top else 1.0
+    if keep < groups:
+        gs = torch.sort(best, descending=True).values
+        margin = min(margin, float(gs[keep - 1] - gs[keep]))
+    return idx, w / (w.sum() + 1e-20), margin
 
 
 def moe_ff(h, mlp, st, p, margins=None):
@@ -113,10 +120,9 @@ def moe_ff(h, mlp, st, p, margins=None):
     for t in range(h.shape[0]):
         # the router reads the 32-bit rounding of its input, like everything the model sees
         z = st[p + "router"].to(F64) @ h[t]
-        idx, w, masked = route(z, corr, top, groups, keep)
+        idx, w, margin = route(z, corr, top, groups, keep)
         if margins is not None:
-            srt = torch.sort(masked, descending=True).values
-            margins.append(float(srt[top - 1] - srt[top]) if srt.shape[0] > top else 1.0)
+            margins.append(margin)
         for e, we in zip(idx.tolist(), w):
             out[t] += we * (h[t] if e >= E else glu(h[t], st, f"{p}e{e}.", silu))
     if mlp.get("shared"):
