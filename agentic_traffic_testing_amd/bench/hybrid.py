@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the hybrid decoders (Ledazen, Soselix, Semezen) next to the
+"""Prefill and decode throughput of the hybrid decoders (Ledazen, Soselix, Semezen, Lovapel) next to the
 models of the same layer geometry - Llama, and for Soselix and Semezen also the closest earlier
 hybrid family (softmax + recurrent mixers on the same cache and kernels) - through the serving
 engine (scheduler, paged cache / state slots, kernels).
@@ -6,7 +6,7 @@ engine (scheduler, paged cache / state slots, kernels).
 Random-init weights, synthetic token ids.  Per model and shape:
   prefill  - B prompts of P tokens admitted together, one generated token each: prompt tok/s
   decode   - the same B sequences generating N more tokens: generated tok/s
-``python bench.py --hybrid [ledazen|soselix|semezen]`` prints one JSON line per measurement.
+``python bench.py --hybrid [ledazen|soselix|semezen|lovapel]`` prints one JSON line per measurement.
 """
 from __future__ import annotations
 
@@ -23,7 +23,10 @@ SOSELIX = (("soselix-small", "ledazen-small", "small"),
 SEMEZEN = (("semezen-small", "soselix-small", "small"),
            ("semezen-3b-slice", "soselix-3b-slice", "llama-3b-slice"),
            ("semezen-8b-slice", "soselix-8b-slice", "llama-8b-slice"))
-FAMILIES = {"ledazen": PAIRS, "soselix": SOSELIX, "semezen": SEMEZEN}
+LOVAPEL = (("lovapel-small", "semezen-small", "small"),
+           ("lovapel-3b-slice", "semezen-3b-slice", "llama-3b-slice"),
+           ("lovapel-8b-slice", "semezen-8b-slice", "llama-8b-slice"))
+FAMILIES = {"ledazen": PAIRS, "soselix": SOSELIX, "semezen": SEMEZEN, "lovapel": LOVAPEL}
 
 
 def _engine(model: str, device: str, dtype: str, max_len: int, seqs: int, budget: int):

@@ -44,7 +44,6 @@ namespace mixk {
 constexpr int kMoeRows = 64;        // rows per tile
 constexpr int kMoeFeat = 64;        // output features per workgroup
 constexpr int kMaxExperts = 1024;
-constexpr int kRoutePer = kMaxExperts / kWave;
 
 __device__ __forceinline__ void wave_argmax(float& best, int& be) {
 #pragma unroll
@@ -60,22 +59,24 @@ __device__ __forceinline__ void wave_argmax(float& best, int& be) {
 
 // Every wave runs to the end (rows past T_ recompute the last row and write nothing), so the
 // workgroup barriers around the LDS exchange of the grouped form are reached by all of them.
+// PER: experts per lane (64 PER >= E), so few experts cost few registers, LDS and instructions.
+template <int PER>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
                  const float* __restrict__ correction, int T_, int E, int top, int softmax,
                  int groups, int keep, int renorm) {
-  __shared__ float s_choice[4][kMaxExperts];
-  __shared__ unsigned char s_kept[4][kMaxExperts];
+  __shared__ float s_choice[4][PER * kWave];
+  __shared__ unsigned char s_kept[4][PER * kWave];
   const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t_raw = blockIdx.x * 4 + wv;
   const bool live = t_raw < T_;
   const int t = live ? t_raw : T_ - 1;
   const float* row = logits + static_cast<int64_t>(t) * E;
-  float sc[kRoutePer], ch[kRoutePer];
-  int pick[kRoutePer];
+  float sc[PER], ch[PER];
+  int pick[PER];
   float zmax = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < kRoutePer; ++j) {
+  for (int j = 0; j < PER; ++j) {
     const int e = lane + j * kWave;
     sc[j] = e < E ? row[e] : -INFINITY;
     zmax = fmaxf(zmax, sc[j]);
@@ -86,34 +87,34 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
     for (int o = 32; o > 0; o >>= 1) zmax = fmaxf(zmax, __shfl_xor(zmax, o, kWave));
     float sum = 0.f;
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) {
+    for (int j = 0; j < PER; ++j) {
       sc[j] = lane + j * kWave < E ? expf(sc[j] - zmax) : 0.f;
       sum += sc[j];
     }
     sum = wave_sum(sum);
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) sc[j] = sc[j] / sum;
+    for (int j = 0; j < PER; ++j) sc[j] = sc[j] / sum;
   } else {
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) sc[j] = sigmoidf_(sc[j]);
+    for (int j = 0; j < PER; ++j) sc[j] = sigmoidf_(sc[j]);
   }
 #pragma unroll
-  for (int j = 0; j < kRoutePer; ++j) {
+  for (int j = 0; j < PER; ++j) {
     const int e = lane + j * kWave;
     ch[j] = e < E ? sc[j] + (correction != nullptr ? correction[e] : 0.f) : -INFINITY;
   }
   if (groups > 1) {   // uniform over the launch
     const int gs = E / groups;
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int e = lane + j * kWave;
       if (e < E) s_choice[wv][e] = ch[j];
       if (e < groups) s_kept[wv][e] = 0;
     }
     __syncthreads();
-    float gm[kRoutePer];
+    float gm[PER];
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int g = lane + j * kWave;
       gm[j] = -INFINITY;
       if (g < groups)
@@ -123,14 +124,14 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
       float best = -INFINITY;
       int be = 0x7fffffff;
 #pragma unroll
-      for (int j = 0; j < kRoutePer; ++j)
+      for (int j = 0; j < PER; ++j)
         if (gm[j] > best) {
           best = gm[j];
           be = lane + j * kWave;
         }
       wave_argmax(best, be);
 #pragma unroll
-      for (int j = 0; j < kRoutePer; ++j)
+      for (int j = 0; j < PER; ++j)
         if (lane + j * kWave == be) {
           gm[j] = -INFINITY;
           s_kept[wv][be] = 1;
@@ -138,7 +139,7 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int e = lane + j * kWave;
       if (e < E && !s_kept[wv][e / gs]) ch[j] = -INFINITY;
     }
@@ -147,7 +148,7 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
     float best = -INFINITY;
     int be = 0x7fffffff;
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j)
+    for (int j = 0; j < PER; ++j)
       if (ch[j] > best) {   // ascending e inside a lane: the first of equals wins
         best = ch[j];
         be = lane + j * kWave;
@@ -161,7 +162,7 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
       continue;
     }
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j)
+    for (int j = 0; j < PER; ++j)
       if (lane + j * kWave == be) {
         ch[j] = -INFINITY;
         pick[j] = k;
@@ -169,12 +170,12 @@ moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __
   }
   float tot = 0.f;
 #pragma unroll
-  for (int j = 0; j < kRoutePer; ++j)
+  for (int j = 0; j < PER; ++j)
     if (pick[j] >= 0) tot += sc[j];
   tot = wave_sum(tot);
   if (!live) return;
 #pragma unroll
-  for (int j = 0; j < kRoutePer; ++j)
+  for (int j = 0; j < PER; ++j)
     if (pick[j] >= 0) {
       idx[static_cast<int64_t>(t) * top + pick[j]] = lane + j * kWave;
       wts[static_cast<int64_t>(t) * top + pick[j]] = renorm ? sc[j] / (tot + 1e-20f) : sc[j];
@@ -626,8 +627,16 @@ extern "C" int mixk_moe_route(int* idx, float* wts, const float* logits, const f
   if (E < 1 || E > kMaxExperts || top < 1 || top > E || groups < 1 || E % groups != 0 ||
       keep < 1 || keep > groups || top > keep * (E / groups))
     return -1;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T_ + 3) / 4), dim3(256), 0, st, idx, wts, logits,
-                     correction, T_, E, top, softmax, groups, keep, renorm);
+#define MIXK_ROUTE(PER)                                                                          \
+  hipLaunchKernelGGL(moe_route_kernel<PER>, dim3((T_ + 3) / 4), dim3(256), 0, st, idx, wts,      \
+                     logits, correction, T_, E, top, softmax, groups, keep, renorm)
+  if (E <= kWave)
+    MIXK_ROUTE(1);
+  else if (E <= 4 * kWave)
+    MIXK_ROUTE(4);
+  else
+    MIXK_ROUTE(kMaxExperts / kWave);
+#undef MIXK_ROUTE
   return static_cast<int>(hipGetLastError());
 }
 

@@ -132,7 +132,7 @@ def parse_args(argv=None):
     ap.add_argument("--max-tokens-limit", type=int, default=0,
                     help="--via http: clamp every LLM call's max_tokens (0 = off)")
     ap.add_argument("--hybrid", nargs="?", const="ledazen", default="",
-                    choices=["ledazen", "soselix", "semezen"],
+                    choices=["ledazen", "soselix", "semezen", "lovapel"],
                     help="instead of the headline workload: prefill / decode tok/s of a hybrid "
                          "family's presets (default ledazen) next to the presets of the same "
                          "layer geometry of the other families (bench/hybrid.py), one JSON line "
