@@ -574,3 +574,157 @@ def test_moe_experts(dt, T, E, top, ff, W):
         finally:
             mx.MOE_LIBRARY_FLOPS = old
         assert torch.allclose(got.cpu().float(), want.float(), **t), library_from
+
+
+# ---- sandwich-norm boundary, whole-projection q / k norm, grouped routing, SiLU-GLU experts ----
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("W", [96, 100, 1024, 4096, 20000])
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+def test_norm_add_norm(dt, W, kind):
+    """Vector and plain kernel, both norms; rows with a common offset so the mean matters; every
+    combination of (branch added or not) x (next norm or not) that a model uses."""
+    torch.manual_seed(18)
+    T = 7
+    x = torch.randn(T, W) * 2 + 3
+    y = (torch.randn(T, W) * 5 - 20).to(dt)
+    wp, wn = (torch.rand(W) + 0.5).to(dt), (torch.rand(W) + 0.5).to(dt)
+    t = dict(atol=4e-2, rtol=2e-2) if dt == torch.bfloat16 else dict(atol=3e-5, rtol=3e-5)
+    for add, nxt in ((True, True), (False, True), (True, False)):
+        xr, xg = x.clone(), x.clone().cuda()
+        hr = mref.norm_add_norm(xr, y if add else None, wp if add else None, wn if nxt else None,
+                                1e-5, kind == "layer", dt)
+        hg = mx.norm_add_norm(xg, y.cuda() if add else None, wp.cuda() if add else None,
+                              wn.cuda() if nxt else None, 1e-5, kind, dt)
+        assert torch.allclose(xg.cpu(), xr, atol=3e-5, rtol=3e-5), (add, nxt)
+        assert (hg is None) == (hr is None)
+        if nxt:
+            assert torch.allclose(hg.cpu().float(), hr.float(), **t), (add, nxt)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,vdim,rot", [(6, 2, 64, 48, 24), (4, 1, 48, 48, 48),
+                                               (8, 2, 128, 128, 64), (3, 3, 10, 6, 0)])
+def test_whole_projection_norm_front_end(dt, H, G, dim, vdim, rot):
+    """q and k normed over all their heads at once with weights per row of the projection
+    (slices of a fused projection, aligned and not), then rotate-half positions."""
+    torch.manual_seed(19)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, nb, bs = int(md["seq_qstart"][-1]), md["num_pages"], 16
+    nq, nk, nv = H * dim, G * dim, G * vdim
+    P = torch.randn(T, nq + nk + nv + 16).to(dt)
+    P[:, 8:8 + dim] *= 20                         # one large head: a per-head norm would differ
+    sq = (slice(None), slice(8, 8 + nq))
+    sk = (slice(None), slice(8 + nq, 8 + nq + nk))
+    sv = (slice(None), slice(8 + nq + nk, 8 + nq + nk + nv))
+    qw, kw = (torch.rand(nq) + 0.5).to(dt), (torch.rand(nk) + 0.5).to(dt)
+    tab = (mref.rotary_table(md["positions"], mx.inv_freq(rot, 30000.0, "cpu")) if rot else
+           torch.zeros(T, 0))
+    kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, vdim, bs).to(dt)
+    kcg, vcg, Pg = kc.cuda(), vc.cuda(), P.cuda()
+    qr = mref.qk_norm_rope_cache(P[sq], P[sk], P[sv], qw, kw, 1e-6, md["positions"],
+                                 md["slot_mapping"], tab, kc, vc, H, G, dim, vdim, True, False, True)
+    qg = mx.qk_norm_rope_cache(Pg[sq], Pg[sk], Pg[sv], qw.cuda(), kw.cuda(), 1e-6,
+                               mdg["positions"], mdg["slot_mapping"], tab.cuda(), kcg, vcg, H, G,
+                               dim, vdim, rotate_half_pairs=True, whole_norm=True)
+    assert torch.allclose(qg.cpu().float(), qr.float(), **tol(dt))
+    assert torch.allclose(kcg.cpu().float(), kc.float(), **tol(dt))
+    assert torch.equal(vcg.cpu(), vc)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("window", [0, 40, 128])
+def test_learned_sink_with_window(dt, window):
+    """The per-head sink score together with a window, in prefill tiles and in decode rows whose
+    window covers one or several partitions (the combine adds the sink once)."""
+    torch.manual_seed(20)
+    H, G, dim, vdim = 6, 2, 64, 64
+    lens, starts = [1, 1, 1, 150, 70], [0, 130, 700, 333, 0]
+    md = ragged(lens, starts, list(range(5)), width=64)
+    keep = md["tile_seq"] >= 3
+    md["tile_seq"], md["tile_qoff"] = md["tile_seq"][keep], md["tile_qoff"][keep]
+    mdg = cuda(md)
+    T, nb = int(md["seq_qstart"][-1]), md["num_pages"]
+    q = torch.randn(T, H, dim).to(dt)
+    kc, vc = torch.randn(nb, G, 16, dim).to(dt), torch.randn(nb, G, vdim, 16).to(dt)
+    sink = torch.tensor([-20.0, -1.0, 0.0, 2.0, 6.0, 30.0])
+    want = mref.sink_attention(q, kc, vc, md["block_tables"], md["seq_kvlen"], md["seq_qstart"],
+                               0.15, True, sink, window)
+    for mfma in (True, False):
+        mx.ATTENTION_MFMA = mfma
+        try:
+            got = mx.sink_attention(q.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                    mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                    mdg["tile_qoff"], 0.15, True, num_decode=3, max_decode_kv=701,
+                                    sink_values=sink.cuda(), window=window)
+        finally:
+            mx.ATTENTION_MFMA = True
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt)), (mfma, window)
+
+
+@pytest.mark.parametrize("E,top,groups,keep", [(10, 1, 1, 1), (18, 4, 3, 2), (64, 6, 8, 3),
+                                               (70, 4, 5, 2), (256, 8, 8, 4), (300, 5, 300, 7),
+                                               (1024, 8, 16, 2), (3, 3, 3, 3)])
+@pytest.mark.parametrize("softmax", [True, False])
+def test_moe_route_grouped(E, top, groups, keep, softmax):
+    """All three register tiers of the route kernel (<= 64, <= 256, <= 1024 experts), row counts
+    that leave waves of the last workgroup without a row, with and without correction."""
+    torch.manual_seed(21)
+    for T in (1, 6, 203):
+        logits = torch.randn(T, E) * 3
+        corr = torch.randn(E) * (0.3 / E if softmax else 0.2)
+        for c in (corr, None):
+            for renorm in (True, False):
+                idx, wts = mx.moe_route(logits.cuda(), top, "softmax" if softmax else "sigmoid",
+                                        None if c is None else c.cuda(), groups, keep, renorm)
+                ri, rw = mref.moe_route(logits, top, softmax, c, groups, keep, renorm)
+                # the order among the chosen is by choice score; compare as sets with weights
+                so, ro = torch.argsort(idx.cpu(), 1), torch.argsort(ri, 1)
+                same = (torch.gather(idx.cpu(), 1, so) == torch.gather(ri, 1, ro)).all(1)
+                assert same.float().mean() > 0.97     # fp32 ties between near-equal scores aside
+                gw, ww = torch.gather(wts.cpu(), 1, so), torch.gather(rw, 1, ro)
+                assert torch.allclose(gw[same], ww[same], atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("T,E,ident,top,ff,W", [(150, 10, 0, 1, 72, 328), (3, 6, 2, 2, 48, 96),
+                                                (700, 4, 1, 2, 200, 136), (65, 5, 3, 3, 30, 50),
+                                                (1, 8, 0, 1, 128, 256), (5, 6, 2, 2, 1024, 128),
+                                                (2, 1, 3, 2, 584, 64)])
+def test_moe_experts_silu_identity(dt, T, E, ident, top, ff, W):
+    """The SiLU-GLU form with the weights on the outputs, identity experts and an added row, in
+    all tile forms of the grouped kernels (small, large, split down product, rows kernels) and on
+    the library path."""
+    torch.manual_seed(22)
+    h = torch.randn(T, W).to(dt)
+    wgu = (torch.randn(E, 2 * ff, W) * 2 / W ** 0.5).to(dt)
+    wd = (torch.randn(E, W, ff) / ff ** 0.5).to(dt)
+    idx, wts = mref.moe_route(torch.randn(T, E + ident) * 2, top, True, None, 1, 1, True)
+    add = torch.randn(T, W).to(dt)
+    t = dict(atol=6e-2, rtol=3e-2) if dt == torch.bfloat16 else dict(atol=5e-5, rtol=5e-5)
+    for addend in (add, None):
+        want = mref.moe_experts(h, idx, wts, wgu, wd, 0.0, 0.0, True, addend)
+        for library_from in (0, 1):
+            old, mx.MOE_LIBRARY_FLOPS = mx.MOE_LIBRARY_FLOPS, library_from
+            try:
+                got = mx.moe_experts(h.cuda(), idx.cuda(), wts.cuda(), wgu.cuda(), wd.cuda(),
+                                     glu="silu", addend=None if addend is None else addend.cuda())
+            finally:
+                mx.MOE_LIBRARY_FLOPS = old
+            assert torch.allclose(got.cpu().float(), want.float(), **t), library_from
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_strided_glu_and_softcap(dt):
+    torch.manual_seed(23)
+    for T, n, pad in ((5, 72, 8), (3, 50, 6), (300, 1024, 0)):
+        P = (torch.randn(T, 2 * n + pad) * 3).to(dt)
+        g, u = P[:, :n], P[:, n + pad:]
+        for act, code in (("gelu_tanh", 2), ("silu", 0), ("sigmoid", 1)):
+            got = mx.gate_mul(P.cuda()[:, n + pad:], P.cuda()[:, :n], act)
+            assert torch.allclose(got.cpu().float(), mref.gate_mul(u, g, code).float(), **tol(dt))
+    z = (torch.randn(9, 1000) * 40).to(dt)
+    for scale, cap in ((0.25, 15.0), (1.0, 0.0), (2.0, 50.0)):
+        got = mx.scale_softcap(z.cuda(), scale, cap)
+        assert got.dtype == torch.float32
+        assert torch.allclose(got.cpu(), mref.scale_softcap(z, scale, cap), atol=2e-5, rtol=1e-5)
