@@ -226,7 +226,7 @@ def test_other_sizes(model_dir, device):
                            "shared": {"ff": 7}}),
         "wide": dict(order="ed", width=64, ff=72, loop=(1, 2, 2),
                      att={"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.11,
-                          "mask": {"size": 64}, "rot": {"dims": 64, "base": 20000.0}},
+                          "mask": {"size": 64}, "rot": {"dims": 64, "base": 15000.0}},
                      moe={"kind": "moe", "expert": {"ff": 32},
                           "router": {"experts": 6, "identity": 2, "top": 2,
                                      "groups": {"count": 4, "keep": 3}},
@@ -476,7 +476,8 @@ def attend(q, kc, vc, bt, T, n, window, scale, sink, device, decode=False):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, pytest.param(torch.bfloat16, marks=pytest.mark.gpu)])
-@pytest.mark.parametrize("T,window", [(300, 72), (129, 128), (200, 17), (64, 200)])
+@pytest.mark.parametrize("T,window", [(300, 75), (129, 128), (200, 17), (64, 200), (700, 0),
+                                      (700, 690)])
 def test_window_edge_and_sink(device, dtype, T, window):
     """One key stands out by its score: it decides the output while it is the oldest key of the
     window and is gone one row later, in prompts and in decoding, across page and partition
@@ -488,7 +489,9 @@ def test_window_edge_and_sink(device, dtype, T, window):
     k = 0.05 * torch.randn(T, G, d, generator=g)
     v = torch.randn(T, G, dv, generator=g)
     q = 0.05 * torch.randn(T, H, d, generator=g)
-    j = max(0, T - window - 3)                      # the marked key
+    # the marked key: three rows before the last window begins; with no window or a long one it
+    # lies hundreds of keys back, on the first page
+    j = max(0, T - window - 3) if 0 < window < 600 else 5
     k[j] = 0.0
     k[j, :, 0] = 9.0
     q[:, :, 0] = 3.0                                # score 27 against the marked key, ~0 otherwise
@@ -502,7 +505,7 @@ def test_window_edge_and_sink(device, dtype, T, window):
     got = attend(q[T - n:], kc, vc, bt, T, n, window, 1.0, sink, device)
     tol = dict(atol=2e-3, rtol=2e-3) if dtype == torch.float32 else dict(atol=0.6, rtol=3e-2)
     assert torch.allclose(got.double(), want[T - n:], **tol)
-    last_in = j + window - 1                        # the last row that still sees the marked key
+    last_in = j + window - 1 if window else T - 1   # the last row that still sees the marked key
     if last_in < T:
         assert got[last_in - (T - n), 1].mean() > 90 and got[last_in - (T - n), 2].mean() < 60
         if last_in + 1 < T:

@@ -662,7 +662,7 @@ def test_learned_sink_with_window(dt, window):
         assert torch.allclose(got.cpu().float(), want.float(), **tol(dt)), (mfma, window)
 
 
-@pytest.mark.parametrize("E,top,groups,keep", [(10, 1, 1, 1), (18, 4, 3, 2), (64, 6, 8, 3),
+@pytest.mark.parametrize("E,top,groups,keep", [(10, 1, 1, 1), (20, 3, 5, 2), (64, 6, 8, 3),
                                                (70, 4, 5, 2), (256, 8, 8, 4), (300, 5, 300, 7),
                                                (1024, 8, 16, 2), (3, 3, 3, 3)])
 @pytest.mark.parametrize("softmax", [True, False])
@@ -724,7 +724,7 @@ def test_strided_glu_and_softcap(dt):
             got = mx.gate_mul(P.cuda()[:, n + pad:], P.cuda()[:, :n], act)
             assert torch.allclose(got.cpu().float(), mref.gate_mul(u, g, code).float(), **tol(dt))
     z = (torch.randn(9, 1000) * 40).to(dt)
-    for scale, cap in ((0.25, 15.0), (1.0, 0.0), (2.0, 50.0)):
+    for scale, cap in ((0.3, 12.0), (1.0, 0.0), (2.0, 50.0)):
         got = mx.scale_softcap(z.cuda(), scale, cap)
         assert got.dtype == torch.float32
         assert torch.allclose(got.cpu(), mref.scale_softcap(z, scale, cap), atol=2e-5, rtol=1e-5)
