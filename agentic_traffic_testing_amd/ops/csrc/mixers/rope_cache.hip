@@ -53,7 +53,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
   T* dst = is_q ? q_out + (static_cast<int64_t>(t) * H + head) * dim
                 : k_cache + ((static_cast<int64_t>(slot / block_size) * G + (head - H)) *
                                  block_size + slot % block_size) * dim;
-  const int pairs = dim >> 1;
+  const int pairs = (dim + 1) >> 1;   // an odd width leaves the last pair half empty
   const float* tab = cos_sin + static_cast<int64_t>(t) * 2 * n_freq;   // [cos | sin] of row t
   float u[kMaxPairs], v[kMaxPairs];
   float ss = 0.f;
@@ -65,7 +65,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
       // pair i: channels (2i, 2i + 1), or (i, i + n_freq) for the rotated ones of the half layout
       const int ca = (half && i < n_freq) ? i : 2 * i, cb = (half && i < n_freq) ? i + n_freq : 2 * i + 1;
       u[j] = ldf(src + ca);
-      v[j] = ldf(src + cb);
+      v[j] = cb < dim ? ldf(src + cb) : 0.f;
       if (norm_last && i < n_freq) {
         const float cs = tab[i], sn = tab[n_freq + i];
         const float ra = u[j] * cs - v[j] * sn;
@@ -88,7 +88,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
     if (i >= pairs) continue;
     const int ca = (half && i < n_freq) ? i : 2 * i, cb = (half && i < n_freq) ? i + n_freq : 2 * i + 1;
     float a = u[j] * inv * (w != nullptr ? ldf(w + ca) : 1.0f);
-    float b = v[j] * inv * (w != nullptr ? ldf(w + cb) : 1.0f);
+    float b = v[j] * inv * (w != nullptr && cb < dim ? ldf(w + cb) : 1.0f);
     if (!norm_last && i < n_freq) {
       const float cs = tab[i], sn = tab[n_freq + i];
       const float ra = a * cs - b * sn;
@@ -97,7 +97,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
       b = rb;
     }
     stf(dst + ca, a);
-    stf(dst + cb, b);
+    if (cb < dim) stf(dst + cb, b);
   }
 }
 
@@ -213,7 +213,7 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                        int block_size, int half, int norm_last,
                                        const float* row_inv, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
-  if (dim > 2 * kWave * kMaxPairs || (dim & 1) || (row_inv != nullptr && norm_last)) return -1;
+  if (dim > 2 * kWave * kMaxPairs || (row_inv != nullptr && norm_last)) return -1;
   MIXK_DISPATCH(dtype,
                 hipLaunchKernelGGL(v_cache_write_kernel<T>, dim3((T_ + 7) / 8, G), dim3(128), 0,
                                    st, static_cast<const T*>(vx), v_stride, slot_mapping,

@@ -204,7 +204,7 @@ def test_other_sizes(model_dir, device):
     heads; rotation of the whole head and none; no window and a window of one key; one group and
     groups of one expert; every route chosen and a single one; no identity experts, no shared
     expert; only identity experts besides one; no loop, a loop over everything, a loop that
-    runs once; no soft cap; widths that are not multiples of 8."""
+    runs once; no soft cap; widths that are not multiples of 8, odd head widths."""
     variants = {
         "one": dict(order="-e-", width=40, loop=(0, 3, 3), cap=0.0, scale=1.0,
                     att={"heads": 3, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 0.3,
@@ -224,6 +224,9 @@ def test_other_sizes(model_dir, device):
                            "router": {"experts": 1, "identity": 3, "top": 2,
                                       "groups": {"count": 2, "keep": 1}},
                            "shared": {"ff": 7}}),
+        "odd": dict(order="d", width=30, ff=11, loop=None,
+                    att={"heads": 2, "kv_heads": 1, "dim": 9, "vdim": 5, "scale": 0.3,
+                         "mask": {"size": 40}, "rot": {"dims": 4, "base": 50.0}}),
         "wide": dict(order="ed", width=64, ff=72, loop=(1, 2, 2),
                      att={"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.11,
                           "mask": {"size": 64}, "rot": {"dims": 64, "base": 15000.0}},

@@ -603,7 +603,8 @@ def test_norm_add_norm(dt, W, kind):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,G,dim,vdim,rot", [(6, 2, 64, 48, 24), (4, 1, 48, 48, 48),
-                                               (8, 2, 128, 128, 64), (3, 3, 10, 6, 0)])
+                                               (8, 2, 128, 128, 64), (3, 3, 10, 6, 0),
+                                               (3, 1, 9, 5, 4)])
 def test_whole_projection_norm_front_end(dt, H, G, dim, vdim, rot):
     """q and k normed over all their heads at once with weights per row of the projection
     (slices of a fused projection, aligned and not), then rotate-half positions."""
